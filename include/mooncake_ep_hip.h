@@ -1,0 +1,169 @@
+/*
+ * C ABI of libmooncake_ep_hip.so: mooncake-ep's low-latency MoE dispatch /
+ * combine for one AMD MI355X (gfx950), with the expert-parallel world kept as
+ * logical ranks inside that GPU's HBM.
+ *
+ * The entry points are what the reference's Python binding for this path
+ * binds (mooncake-ep/src/ep_py.cpp:14-46, class MooncakeEpBuffer in
+ * mooncake-ep/include/mooncake_ep_buffer.h:66-194), flattened to plain
+ * pointers and integers.  Device addresses and streams travel as uint64_t
+ * exactly as in the reference's signatures.  Every function returns 0 on
+ * success or an MC_EP_ERR_* code; mc_ep_last_error() returns the message of
+ * the calling thread's last failure.  The reference raises EPException
+ * ("Failed: Assertion error file:line 'cond'", mooncake_ep_exception.cuh:12-45)
+ * where this ABI returns MC_EP_ERR_ASSERT with the same condition text.
+ *
+ * Not thread-safe per object, like the reference
+ * (mooncake_ep_buffer.cpp:215-218): drive one world from one thread.
+ */
+#ifndef MOONCAKE_EP_HIP_H
+#define MOONCAKE_EP_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MC_EP_OK 0
+#define MC_EP_ERR_ASSERT 1      /* a host assertion of the reference failed */
+#define MC_EP_ERR_HIP 2         /* a HIP runtime call failed */
+#define MC_EP_ERR_PENDING 3     /* a collective is waited on before every live rank has called it */
+#define MC_EP_ERR_UNSUPPORTED 4 /* zero-copy combine etc. (NotImplementedError in the reference) */
+
+/* mooncake_ep_configs.cuh:5 */
+#define MC_EP_MAX_QP_COUNT 256
+
+/* phases of a whole-world call (the reference's LOW_LATENCY_SEND_PHASE /
+ * LOW_LATENCY_RECV_PHASE split, mooncake_ep_configs.cuh:16-17, maps onto the
+ * two kernels each call is made of) */
+#define MC_EP_PHASE_LAYOUT 1   /* dispatch: routing layout;  combine: handle -> row resolve */
+#define MC_EP_PHASE_DATA 2     /* dispatch: pack;            combine: weighted reduce */
+#define MC_EP_PHASE_ALL 3
+
+typedef struct mc_ep_world mc_ep_world_t;     /* R logical ranks on one device */
+typedef struct mc_ep_buffer mc_ep_buffer_t;   /* one rank's MooncakeEpBuffer */
+typedef struct mc_ep_event mc_ep_event_t;     /* EventHandle */
+typedef struct mc_ep_hook mc_ep_hook_t;       /* the recv hook closure */
+
+const char* mc_ep_last_error(void);
+
+/* get_ep_buffer_size_hint, mooncake_ep_buffer.h:197-203 (BufferPair, :29-63) */
+uint64_t mc_ep_get_buffer_size_hint(int num_max_dispatch_tokens_per_rank, int hidden, int num_ranks,
+                                    int num_experts);
+
+/* ---- the logical world ------------------------------------------------- */
+
+/* Replaces process-group bootstrap + peer exchange (Buffer.__init__/connect,
+ * mooncake-wheel/mooncake/mooncake_ep_buffer.py:93-119,185-304): all ranks
+ * share one address space, so there is nothing to exchange.  Uses the
+ * calling thread's current HIP device. */
+int mc_ep_world_create(int num_ranks, mc_ep_world_t** out);
+int mc_ep_world_destroy(mc_ep_world_t* world);
+int mc_ep_world_num_ranks(const mc_ep_world_t* world);
+
+/* A silent rank never calls dispatch/combine again (the reference's failed
+ * process, mooncake-ep/tests/test_ep_grid.py:121-158); collectives complete
+ * without it.  Forces from the host what the reference detects by timeout
+ * (mooncake_ep_kernel.cu:417-429, :688-698). */
+int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
+
+/* Tuning knobs for measurement sweeps ("pack_variant", "pack_waves",
+ * "combine_chunks", "combine_waves", "layout_block", "nontemporal",
+ * "scale_mode"). */
+int mc_ep_world_set_option(mc_ep_world_t* world, const char* name, int value);
+int mc_ep_world_get_option(const mc_ep_world_t* world, const char* name, int* value);
+
+/* Whole-world dispatch: every rank's MooncakeEpBuffer::dispatch
+ * (mooncake_ep_buffer.h:116-124, mooncake_ep_buffer.cpp:193-339) in one
+ * launch sequence on `stream_ptr`.  Each *_ptrs argument is a host array of
+ * num_ranks device addresses (rank r's tensor); num_tokens is a host array.
+ * A rank with packed_recv_x_ptrs[r] == 0 receives nothing; a rank with
+ * num_tokens[r] == 0 sends nothing.  packed_recv_x_scales_ptrs may be NULL
+ * when use_fp8 == 0.  Tensor shapes per rank as in the reference:
+ *   x [T_r, hidden] bf16, topk_idx [T_r, num_topk] int64,
+ *   packed_recv_x [E/R, R*max, hidden] fp8 e4m3fn | bf16,
+ *   packed_recv_x_scales [E/R, hidden/128, R*max] f32 (physical layout),
+ *   packed_recv_count [E/R] int32, packed_recv_src_info [E/R, R*max] int32,
+ *   packed_recv_layout_range [E/R, R] int64. */
+int mc_ep_world_dispatch(mc_ep_world_t* world, const uint64_t* x_ptrs, const uint64_t* topk_idx_ptrs,
+                         const int32_t* num_tokens, int hidden, int num_topk,
+                         int num_max_dispatch_tokens_per_rank, int num_experts, int use_fp8,
+                         const uint64_t* packed_recv_x_ptrs, const uint64_t* packed_recv_x_scales_ptrs,
+                         const uint64_t* packed_recv_count_ptrs, const uint64_t* packed_recv_src_info_ptrs,
+                         const uint64_t* packed_recv_layout_range_ptrs, int phases, uint64_t stream_ptr);
+
+/* Whole-world combine: every rank's MooncakeEpBuffer::combine
+ * (mooncake_ep_buffer.h:126-133, mooncake_ep_buffer.cpp:341-474).
+ *   x [E/R, R*max, hidden] bf16 (expert outputs held by the rank; 0: the rank
+ *   contributes nothing), topk_idx / topk_weights [T_r, num_topk],
+ *   src_info / layout_range: the handle returned by that rank's dispatch,
+ *   active_ranks [R] int32 (rank r's own view), combined_x [T_r, hidden] bf16. */
+int mc_ep_world_combine(mc_ep_world_t* world, const uint64_t* x_ptrs, const uint64_t* topk_idx_ptrs,
+                        const uint64_t* topk_weights_ptrs, const uint64_t* src_info_ptrs,
+                        const uint64_t* layout_range_ptrs, const uint64_t* active_ranks_ptrs,
+                        const int32_t* num_combined_tokens, int hidden, int num_topk,
+                        int num_max_dispatch_tokens_per_rank, int num_experts, const uint64_t* combined_x_ptrs,
+                        int phases, uint64_t stream_ptr);
+
+/* ---- per-rank Buffer: the reference's binding, one object per rank ------ */
+
+/* MooncakeEpBuffer(rank, num_ranks, num_ep_buffer_bytes, disable_p2p),
+ * ep_py.cpp:27-30.  num_ranks is the world's. */
+int mc_ep_buffer_create(mc_ep_world_t* world, int rank, int64_t num_ep_buffer_bytes, int disable_p2p,
+                        mc_ep_buffer_t** out);
+int mc_ep_buffer_destroy(mc_ep_buffer_t* buffer);
+
+/* Transport introspection (ep_py.cpp:31-42).  One GPU: no NIC, every peer is
+ * in the same address space. */
+int mc_ep_buffer_ibgda_disabled(const mc_ep_buffer_t* buffer);   /* 1 */
+int mc_ep_buffer_p2p_enabled(const mc_ep_buffer_t* buffer);      /* !disable_p2p */
+int mc_ep_buffer_use_fast_path(const mc_ep_buffer_t* buffer);    /* 1 */
+int mc_ep_buffer_is_roce(const mc_ep_buffer_t* buffer);          /* 0 */
+
+/* MooncakeEpBuffer::dispatch, argument order of mooncake_ep_buffer.h:116-124.
+ * Dispatch is a collective over the world's live ranks: the call records this
+ * rank's arguments, and the call that completes the round launches the
+ * kernels for all ranks.  *event_out is set when async != 0, *hook_out when
+ * return_recv_hook != 0 (else NULL); async together with return_recv_hook is
+ * rejected (mooncake_ep_buffer.cpp:226). */
+int mc_ep_buffer_dispatch(mc_ep_buffer_t* buffer, uint64_t x_ptr, uint64_t topk_idx_ptr, uint64_t active_ranks_ptr,
+                          int num_tokens, int hidden, int num_topk, int num_max_dispatch_tokens_per_rank,
+                          int num_experts, int timeout_us, int use_fp8, uint64_t packed_recv_x_ptr,
+                          uint64_t packed_recv_x_scales_ptr, uint64_t packed_recv_count_ptr,
+                          uint64_t packed_recv_src_info_ptr, uint64_t packed_recv_layout_range_ptr, int async,
+                          int return_recv_hook, uint64_t compute_stream_ptr, mc_ep_event_t** event_out,
+                          mc_ep_hook_t** hook_out);
+
+/* MooncakeEpBuffer::combine, argument order of mooncake_ep_buffer.h:126-133. */
+int mc_ep_buffer_combine(mc_ep_buffer_t* buffer, uint64_t x_ptr, uint64_t topk_idx_ptr, uint64_t topk_weights_ptr,
+                         uint64_t src_info_ptr, uint64_t layout_range_ptr, uint64_t active_ranks_ptr,
+                         int num_local_experts, int num_combined_tokens, int hidden, int num_topk,
+                         int num_max_dispatch_tokens_per_rank, int num_experts, int timeout_us, int zero_copy,
+                         uint64_t combined_x_ptr, int async, int return_recv_hook, uint64_t compute_stream_ptr,
+                         mc_ep_event_t** event_out, mc_ep_hook_t** hook_out);
+
+/* ---- EventHandle (mooncake_ep_event.h:9-42) and the recv hook ----------- */
+
+/* EventHandle(stream_ptr): an event recorded on that stream now. */
+int mc_ep_event_create(uint64_t stream_ptr, mc_ep_event_t** out);
+int mc_ep_event_current_stream_wait(mc_ep_event_t* event, uint64_t stream_ptr);
+int mc_ep_event_synchronize(mc_ep_event_t* event);
+int mc_ep_event_destroy(mc_ep_event_t* event);
+
+/* The closure returned for return_recv_hook (mooncake_ep_buffer.cpp:330-335):
+ * after it returns, work queued on the rank's compute stream sees the outputs. */
+int mc_ep_hook_call(mc_ep_hook_t* hook);
+int mc_ep_hook_destroy(mc_ep_hook_t* hook);
+
+/* ---- measurement helper -------------------------------------------------- */
+
+/* Plain device copy of `bytes` (multiple of 16): the known-size kernel the
+ * profiler's FETCH_SIZE / WRITE_SIZE readings are scaled against. */
+int mc_ep_debug_copy(uint64_t dst_ptr, uint64_t src_ptr, uint64_t bytes, uint64_t stream_ptr);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MOONCAKE_EP_HIP_H */

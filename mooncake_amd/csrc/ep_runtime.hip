@@ -1,0 +1,735 @@
+// Host runtime behind the C ABI (include/mooncake_ep_hip.h): the logical EP
+// world, per-rank buffers with the reference's call signatures, event and
+// hook objects.  Mirrors the host side of the reference
+// (mooncake-ep/src/mooncake_ep_buffer.cpp:193-474) minus everything that
+// exists only to move bytes between GPUs: there is no communication buffer,
+// no double buffering, no peer bootstrap.
+#include "../../include/mooncake_ep_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <deque>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "ep_kernels.h"
+
+using namespace mcep;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string& msg) {
+    g_last_error = msg;
+    return code;
+}
+
+#define MC_ASSERT(cond)                                                                                        \
+    do {                                                                                                       \
+        if (!(cond))                                                                                           \
+            return fail(MC_EP_ERR_ASSERT, std::string("Failed: Assertion error ") + __FILE__ + ":" +          \
+                                              std::to_string(__LINE__) + " '" #cond "'");                      \
+    } while (0)
+
+#define MC_HIP(cmd)                                                                                            \
+    do {                                                                                                       \
+        hipError_t e_ = (cmd);                                                                                 \
+        if (e_ != hipSuccess)                                                                                  \
+            return fail(MC_EP_ERR_HIP, std::string("Failed: HIP error ") + __FILE__ + ":" +                   \
+                                           std::to_string(__LINE__) + " '" + hipGetErrorString(e_) + "'");    \
+    } while (0)
+
+// One collective call (a "round"): the j-th dispatch (or combine) of every live rank.
+struct Round {
+    bool launched = false;
+    hipEvent_t done = nullptr;
+    ~Round() {
+        if (done) (void)hipEventDestroy(done);
+    }
+};
+
+struct DispatchPost {
+    bool present = false;
+    uint64_t x = 0, topk_idx = 0, active_ranks = 0;
+    int num_tokens = 0, hidden = 0, num_topk = 0, max_tokens = 0, num_experts = 0, timeout_us = -1, use_fp8 = 0;
+    uint64_t recv_x = 0, recv_scales = 0, recv_count = 0, src_info = 0, layout_range = 0;
+    bool async = false, hook = false;
+    hipStream_t stream = nullptr;
+};
+
+struct CombinePost {
+    bool present = false;
+    uint64_t x = 0, topk_idx = 0, topk_weights = 0, src_info = 0, layout_range = 0, active_ranks = 0, out = 0;
+    int num_tokens = 0, hidden = 0, num_topk = 0, max_tokens = 0, num_experts = 0, timeout_us = -1;
+    bool async = false, hook = false;
+    hipStream_t stream = nullptr;
+};
+
+template <typename Post>
+struct PendingRound {
+    std::vector<Post> posts;
+    std::shared_ptr<Round> state;
+};
+
+}  // namespace
+
+struct mc_ep_world {
+    int device = 0;
+    int R = 0;
+    hipStream_t comm_stream = nullptr;
+    uint64_t* d_tbl[2] = {nullptr, nullptr};     // dispatch, combine pointer tables
+    std::vector<uint64_t> tbl_cache[2];           // what the device tables hold
+    int32_t* d_slot[2] = {nullptr, nullptr};     // (rank, token, k) -> packed row
+    size_t slot_cap[2] = {0, 0};
+    void* d_zero_row = nullptr;
+    Tuning tuning;
+    std::vector<char> silent;
+    // per-rank collective bookkeeping
+    std::deque<PendingRound<DispatchPost>> dispatch_rounds;
+    std::deque<PendingRound<CombinePost>> combine_rounds;
+    std::vector<long long> dispatch_calls, combine_calls;   // calls made per rank
+    long long dispatch_base = 0, combine_base = 0;          // index of the front round
+};
+
+struct mc_ep_buffer {
+    mc_ep_world* world = nullptr;
+    int rank = 0;
+    int64_t num_ep_buffer_bytes = 0;
+    bool p2p_enabled = true;
+};
+
+struct mc_ep_event {
+    std::shared_ptr<Round> round;   // deferred: completion of a collective
+    hipEvent_t own = nullptr;       // immediate: recorded at creation
+};
+
+struct mc_ep_hook {
+    std::shared_ptr<Round> round;
+    hipStream_t stream = nullptr;
+};
+
+namespace {
+
+struct DeviceGuard {
+    int prev = -1;
+    bool changed = false;
+    explicit DeviceGuard(int dev) {
+        if (hipGetDevice(&prev) == hipSuccess && prev != dev) changed = (hipSetDevice(dev) == hipSuccess);
+    }
+    ~DeviceGuard() {
+        if (changed) (void)hipSetDevice(prev);
+    }
+};
+
+int ensure_slot_map(mc_ep_world* w, int which, size_t words) {
+    if (words <= w->slot_cap[which]) return MC_EP_OK;
+    // grows only; the old map may still be read by queued kernels
+    MC_HIP(hipDeviceSynchronize());
+    if (w->d_slot[which]) MC_HIP(hipFree(w->d_slot[which]));
+    w->d_slot[which] = nullptr;
+    w->slot_cap[which] = 0;
+    size_t cap = words + words / 2 + 1024;
+    MC_HIP(hipMalloc((void**)&w->d_slot[which], cap * sizeof(int32_t)));
+    w->slot_cap[which] = cap;
+    return MC_EP_OK;
+}
+
+int upload_table(mc_ep_world* w, int which, const std::vector<uint64_t>& tbl, hipStream_t stream) {
+    if (w->tbl_cache[which] == tbl) return MC_EP_OK;
+    MC_HIP(launch_table_write(w->d_tbl[which], tbl.data(), (int)tbl.size(), stream));
+    w->tbl_cache[which] = tbl;
+    return MC_EP_OK;
+}
+
+// the reference's host assertions on shapes (mooncake_ep_buffer.cpp:202-206,
+// :246-251, :351-354; mooncake_ep_kernel.cu:505, :781)
+int check_dims(const mc_ep_world* w, int hidden, int num_topk, int max_tokens, int num_experts) {
+    MC_ASSERT(num_experts > 0 && num_experts % w->R == 0);
+    MC_ASSERT(hidden > 0 && hidden % 16 == 0 && hidden % 128 == 0);
+    MC_ASSERT((size_t)hidden * 2 <= kZeroRowBytes);
+    MC_ASSERT(num_topk > 0 && num_topk <= kMaxTopK);
+    MC_ASSERT(max_tokens > 0);
+    return MC_EP_OK;
+}
+
+int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_idx, const int32_t* num_tokens,
+                        int hidden, int num_topk, int max_tokens, int num_experts, int use_fp8,
+                        const uint64_t* recv_x, const uint64_t* recv_scales, const uint64_t* recv_count,
+                        const uint64_t* src_info, const uint64_t* layout_range, int phases, hipStream_t stream) {
+    const int R = w->R;
+    if (int rc = check_dims(w, hidden, num_topk, max_tokens, num_experts)) return rc;
+    MC_ASSERT(x != nullptr && topk_idx != nullptr && num_tokens != nullptr);
+    MC_ASSERT(recv_x != nullptr && recv_count != nullptr && src_info != nullptr && layout_range != nullptr);
+    if (use_fp8) {
+        MC_ASSERT(((long long)R * max_tokens) % 4 == 0);
+        MC_ASSERT(recv_scales != nullptr);
+    }
+    int tgrid = 0;
+    std::vector<uint64_t> tbl((size_t)DF_COUNT * R, 0);
+    for (int r = 0; r < R; ++r) {
+        MC_ASSERT(num_tokens[r] >= 0 && num_tokens[r] <= max_tokens);
+        MC_ASSERT(num_tokens[r] == 0 || (x[r] != 0 && topk_idx[r] != 0));
+        if (recv_x[r] != 0) {
+            MC_ASSERT(recv_count[r] != 0 && src_info[r] != 0 && layout_range[r] != 0);
+            if (use_fp8) MC_ASSERT(recv_scales[r] != 0);
+        }
+        tbl[DF_X * R + r] = x[r];
+        tbl[DF_TOPK_IDX * R + r] = topk_idx[r];
+        tbl[DF_RECV_X * R + r] = recv_x[r];
+        tbl[DF_RECV_SCALES * R + r] = (use_fp8 && recv_scales) ? recv_scales[r] : 0;
+        tbl[DF_RECV_COUNT * R + r] = recv_count[r];
+        tbl[DF_SRC_INFO * R + r] = src_info[r];
+        tbl[DF_LAYOUT_RANGE * R + r] = layout_range[r];
+        tbl[DF_NUM_TOKENS * R + r] = (uint64_t)num_tokens[r];
+        if (num_tokens[r] > tgrid) tgrid = num_tokens[r];
+    }
+    DeviceGuard guard(w->device);
+    if (int rc = ensure_slot_map(w, 0, (size_t)R * max_tokens * num_topk)) return rc;
+    if (int rc = upload_table(w, 0, tbl, stream)) return rc;
+    Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
+    if (phases & MC_EP_PHASE_LAYOUT) MC_HIP(launch_layout(w->d_tbl[0], w->d_slot[0], d, w->tuning, stream));
+    if ((phases & MC_EP_PHASE_DATA) && tgrid > 0)
+        MC_HIP(launch_pack(w->d_tbl[0], w->d_slot[0], nullptr, d, use_fp8 != 0, w->tuning, stream));
+    return MC_EP_OK;
+}
+
+int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_idx, const uint64_t* topk_weights,
+                       const uint64_t* src_info, const uint64_t* layout_range, const uint64_t* active_ranks,
+                       const int32_t* num_tokens, int hidden, int num_topk, int max_tokens, int num_experts,
+                       const uint64_t* out, int phases, hipStream_t stream) {
+    const int R = w->R;
+    if (int rc = check_dims(w, hidden, num_topk, max_tokens, num_experts)) return rc;
+    MC_ASSERT(x != nullptr && topk_idx != nullptr && topk_weights != nullptr && num_tokens != nullptr);
+    MC_ASSERT(src_info != nullptr && layout_range != nullptr && active_ranks != nullptr && out != nullptr);
+    int tgrid = 0;
+    std::vector<uint64_t> tbl((size_t)CF_COUNT * R, 0);
+    for (int r = 0; r < R; ++r) {
+        MC_ASSERT(num_tokens[r] >= 0 && num_tokens[r] <= max_tokens);
+        if (num_tokens[r] > 0) {
+            MC_ASSERT(topk_idx[r] != 0 && topk_weights[r] != 0);
+            MC_ASSERT(active_ranks[r] != 0);
+            MC_ASSERT(out[r] != 0);
+        }
+        if (x[r] != 0) MC_ASSERT(src_info[r] != 0 && layout_range[r] != 0);
+        tbl[CF_X * R + r] = x[r];
+        tbl[CF_TOPK_IDX * R + r] = topk_idx[r];
+        tbl[CF_TOPK_W * R + r] = topk_weights[r];
+        tbl[CF_SRC_INFO * R + r] = x[r] ? src_info[r] : 0;
+        tbl[CF_LAYOUT_RANGE * R + r] = x[r] ? layout_range[r] : 0;
+        tbl[CF_ACTIVE * R + r] = active_ranks[r];
+        tbl[CF_OUT * R + r] = out[r];
+        tbl[CF_NUM_TOKENS * R + r] = (uint64_t)num_tokens[r];
+        if (num_tokens[r] > tgrid) tgrid = num_tokens[r];
+    }
+    if (tgrid == 0) return MC_EP_OK;
+    DeviceGuard guard(w->device);
+    if (int rc = ensure_slot_map(w, 1, (size_t)R * max_tokens * num_topk)) return rc;
+    if (int rc = upload_table(w, 1, tbl, stream)) return rc;
+    Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
+    if (phases & MC_EP_PHASE_LAYOUT) MC_HIP(launch_resolve(w->d_tbl[1], w->d_slot[1], d, w->tuning, stream));
+    if (phases & MC_EP_PHASE_DATA)
+        MC_HIP(launch_reduce(w->d_tbl[1], w->d_slot[1], w->d_zero_row, d, w->tuning, stream));
+    return MC_EP_OK;
+}
+
+// Streams of a round: run on the callers' stream when they all share one and
+// nobody asked for an event (the reference's hook mode launches there too,
+// mooncake_ep_buffer.cpp:225); otherwise on the world's communication stream,
+// fenced against every caller's stream before and after, as the reference's
+// default mode does (:227, :325-327).
+template <typename Post>
+hipStream_t pick_launch_stream(mc_ep_world* w, const std::vector<Post>& posts, bool* shared) {
+    hipStream_t first = nullptr;
+    bool have = false, same = true, any_async = false;
+    for (const auto& p : posts) {
+        if (!p.present) continue;
+        if (!have) {
+            first = p.stream;
+            have = true;
+        } else if (p.stream != first) {
+            same = false;
+        }
+        any_async |= p.async;
+    }
+    *shared = have && same && !any_async;
+    return *shared ? first : w->comm_stream;
+}
+
+template <typename Post>
+int fence_before(mc_ep_world* w, const std::vector<Post>& posts, hipStream_t launch) {
+    std::vector<hipStream_t> seen;
+    for (const auto& p : posts) {
+        if (!p.present || p.stream == launch) continue;
+        bool dup = false;
+        for (auto s : seen) dup |= (s == p.stream);
+        if (dup) continue;
+        seen.push_back(p.stream);
+        hipEvent_t ev;
+        MC_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        hipError_t e1 = hipEventRecord(ev, p.stream);
+        hipError_t e2 = (e1 == hipSuccess) ? hipStreamWaitEvent(launch, ev, 0) : e1;
+        (void)hipEventDestroy(ev);
+        MC_HIP(e2);
+    }
+    (void)w;
+    return MC_EP_OK;
+}
+
+template <typename Post>
+int fence_after(const std::vector<Post>& posts, hipStream_t launch, Round* round) {
+    MC_HIP(hipEventCreateWithFlags(&round->done, hipEventDisableTiming));
+    MC_HIP(hipEventRecord(round->done, launch));
+    std::vector<hipStream_t> seen;
+    for (const auto& p : posts) {
+        // default mode: the caller's stream waits for the result; async and
+        // hook callers wait through their event / hook
+        if (!p.present || p.async || p.hook || p.stream == launch) continue;
+        bool dup = false;
+        for (auto s : seen) dup |= (s == p.stream);
+        if (dup) continue;
+        seen.push_back(p.stream);
+        MC_HIP(hipStreamWaitEvent(p.stream, round->done, 0));
+    }
+    round->launched = true;
+    return MC_EP_OK;
+}
+
+// A silent source rank has "timed out": each live rank's active_ranks entry
+// for it drops to 0 when that rank asked for a timeout
+// (mooncake_ep_kernel.cu:421-423, :692-694).
+template <typename Post>
+int mark_silent_inactive(mc_ep_world* w, const std::vector<Post>& posts, hipStream_t launch) {
+    for (int r = 0; r < w->R; ++r) {
+        const auto& p = posts[r];
+        if (!p.present || p.timeout_us == -1 || p.active_ranks == 0) continue;
+        for (int j = 0; j < w->R; ++j) {
+            if (posts[j].present) continue;
+            MC_HIP(launch_fill_u32((void*)(p.active_ranks + (uint64_t)j * 4), 0u, 1, launch));
+        }
+    }
+    return MC_EP_OK;
+}
+
+int launch_dispatch_round(mc_ep_world* w, PendingRound<DispatchPost>& pr) {
+    const int R = w->R;
+    const DispatchPost* first = nullptr;
+    for (const auto& p : pr.posts)
+        if (p.present && !first) first = &p;
+    if (!first) return MC_EP_OK;
+    for (const auto& p : pr.posts) {
+        if (!p.present) continue;
+        // every rank of a collective names the same problem shape
+        MC_ASSERT(p.hidden == first->hidden && p.num_topk == first->num_topk);
+        MC_ASSERT(p.max_tokens == first->max_tokens && p.num_experts == first->num_experts);
+        MC_ASSERT(p.use_fp8 == first->use_fp8);
+    }
+    std::vector<uint64_t> x(R, 0), idx(R, 0), rx(R, 0), rs(R, 0), rc(R, 0), si(R, 0), lr(R, 0);
+    std::vector<int32_t> nt(R, 0);
+    for (int r = 0; r < R; ++r) {
+        const auto& p = pr.posts[r];
+        if (!p.present) continue;
+        x[r] = p.x; idx[r] = p.topk_idx; nt[r] = p.num_tokens;
+        rx[r] = p.recv_x; rs[r] = p.recv_scales; rc[r] = p.recv_count; si[r] = p.src_info; lr[r] = p.layout_range;
+    }
+    DeviceGuard guard(w->device);
+    bool shared = false;
+    hipStream_t launch = pick_launch_stream(w, pr.posts, &shared);
+    if (int e = fence_before(w, pr.posts, launch)) return e;
+    if (int e = mark_silent_inactive(w, pr.posts, launch)) return e;
+    if (int e = world_dispatch_impl(w, x.data(), idx.data(), nt.data(), first->hidden, first->num_topk,
+                                    first->max_tokens, first->num_experts, first->use_fp8, rx.data(), rs.data(),
+                                    rc.data(), si.data(), lr.data(), MC_EP_PHASE_ALL, launch))
+        return e;
+    return fence_after(pr.posts, launch, pr.state.get());
+}
+
+int launch_combine_round(mc_ep_world* w, PendingRound<CombinePost>& pr) {
+    const int R = w->R;
+    const CombinePost* first = nullptr;
+    for (const auto& p : pr.posts)
+        if (p.present && !first) first = &p;
+    if (!first) return MC_EP_OK;
+    for (const auto& p : pr.posts) {
+        if (!p.present) continue;
+        MC_ASSERT(p.hidden == first->hidden && p.num_topk == first->num_topk);
+        MC_ASSERT(p.max_tokens == first->max_tokens && p.num_experts == first->num_experts);
+    }
+    std::vector<uint64_t> x(R, 0), idx(R, 0), tw(R, 0), si(R, 0), lr(R, 0), ar(R, 0), out(R, 0);
+    std::vector<int32_t> nt(R, 0);
+    for (int r = 0; r < R; ++r) {
+        const auto& p = pr.posts[r];
+        if (!p.present) continue;
+        x[r] = p.x; idx[r] = p.topk_idx; tw[r] = p.topk_weights; si[r] = p.src_info; lr[r] = p.layout_range;
+        ar[r] = p.active_ranks; out[r] = p.out; nt[r] = p.num_tokens;
+    }
+    DeviceGuard guard(w->device);
+    bool shared = false;
+    hipStream_t launch = pick_launch_stream(w, pr.posts, &shared);
+    if (int e = fence_before(w, pr.posts, launch)) return e;
+    if (int e = mark_silent_inactive(w, pr.posts, launch)) return e;
+    if (int e = world_combine_impl(w, x.data(), idx.data(), tw.data(), si.data(), lr.data(), ar.data(), nt.data(),
+                                   first->hidden, first->num_topk, first->max_tokens, first->num_experts,
+                                   out.data(), MC_EP_PHASE_ALL, launch))
+        return e;
+    return fence_after(pr.posts, launch, pr.state.get());
+}
+
+template <typename Post>
+bool round_complete(const mc_ep_world* w, const PendingRound<Post>& pr) {
+    for (int r = 0; r < w->R; ++r)
+        if (!pr.posts[r].present && !w->silent[r]) return false;
+    return true;
+}
+
+// Launch every leading round that has all its live ranks.
+int drain_dispatch(mc_ep_world* w) {
+    while (!w->dispatch_rounds.empty() && round_complete(w, w->dispatch_rounds.front())) {
+        int e = launch_dispatch_round(w, w->dispatch_rounds.front());
+        w->dispatch_rounds.pop_front();
+        w->dispatch_base++;
+        if (e) return e;
+    }
+    return MC_EP_OK;
+}
+
+int drain_combine(mc_ep_world* w) {
+    while (!w->combine_rounds.empty() && round_complete(w, w->combine_rounds.front())) {
+        int e = launch_combine_round(w, w->combine_rounds.front());
+        w->combine_rounds.pop_front();
+        w->combine_base++;
+        if (e) return e;
+    }
+    return MC_EP_OK;
+}
+
+template <typename Post>
+PendingRound<Post>& round_for_call(mc_ep_world* w, std::deque<PendingRound<Post>>& rounds, long long base,
+                                   long long call_index) {
+    while ((long long)rounds.size() <= call_index - base) {
+        PendingRound<Post> pr;
+        pr.posts.resize(w->R);
+        pr.state = std::make_shared<Round>();
+        rounds.push_back(std::move(pr));
+    }
+    return rounds[(size_t)(call_index - base)];
+}
+
+std::string missing_ranks_message(const char* what) {
+    return std::string("Failed: ") + what +
+           " is a collective over the world's live ranks and not every one of them has called it yet";
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+
+extern "C" {
+
+const char* mc_ep_last_error(void) { return g_last_error.c_str(); }
+
+uint64_t mc_ep_get_buffer_size_hint(int max_tokens, int hidden, int num_ranks, int num_experts) {
+    (void)num_ranks;
+    // two buffers, each: two signalling areas of num_experts ints and two data
+    // areas of num_experts * max_tokens messages of (2 * 16 + hidden * 2) bytes
+    const uint64_t signaling = (uint64_t)num_experts * sizeof(int);
+    const uint64_t data = (uint64_t)num_experts * (uint64_t)max_tokens * (2 * 16 + (uint64_t)hidden * 2);
+    return 4 * signaling + 4 * data;
+}
+
+int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
+    MC_ASSERT(out != nullptr);
+    MC_ASSERT(num_ranks > 0 && num_ranks <= MC_EP_MAX_QP_COUNT);
+    auto w = std::make_unique<mc_ep_world>();
+    w->R = num_ranks;
+    MC_HIP(hipGetDevice(&w->device));
+    MC_HIP(hipStreamCreateWithFlags(&w->comm_stream, hipStreamNonBlocking));
+    for (int i = 0; i < 2; ++i) {
+        const size_t words = (size_t)(i == 0 ? (int)DF_COUNT : (int)CF_COUNT) * num_ranks;
+        MC_HIP(hipMalloc((void**)&w->d_tbl[i], words * sizeof(uint64_t)));
+    }
+    MC_HIP(hipMalloc(&w->d_zero_row, kZeroRowBytes));
+    MC_HIP(hipMemset(w->d_zero_row, 0, kZeroRowBytes));
+    w->silent.assign(num_ranks, 0);
+    w->dispatch_calls.assign(num_ranks, 0);
+    w->combine_calls.assign(num_ranks, 0);
+    *out = w.release();
+    return MC_EP_OK;
+}
+
+int mc_ep_world_destroy(mc_ep_world_t* w) {
+    if (!w) return MC_EP_OK;
+    DeviceGuard guard(w->device);
+    (void)hipDeviceSynchronize();
+    for (int i = 0; i < 2; ++i) {
+        if (w->d_tbl[i]) (void)hipFree(w->d_tbl[i]);
+        if (w->d_slot[i]) (void)hipFree(w->d_slot[i]);
+    }
+    if (w->d_zero_row) (void)hipFree(w->d_zero_row);
+    if (w->comm_stream) (void)hipStreamDestroy(w->comm_stream);
+    delete w;
+    return MC_EP_OK;
+}
+
+int mc_ep_world_num_ranks(const mc_ep_world_t* w) { return w ? w->R : 0; }
+
+int mc_ep_world_set_rank_silent(mc_ep_world_t* w, int rank, int silent) {
+    MC_ASSERT(w != nullptr && rank >= 0 && rank < w->R);
+    w->silent[rank] = silent ? 1 : 0;
+    // rounds that were only waiting for this rank can go now
+    if (int e = drain_dispatch(w)) return e;
+    return drain_combine(w);
+}
+
+static int* option_slot(Tuning& t, const char* name) {
+    if (!strcmp(name, "layout_block")) return &t.layout_block;
+    if (!strcmp(name, "pack_variant")) return &t.pack_variant;
+    if (!strcmp(name, "pack_waves")) return &t.pack_waves;
+    if (!strcmp(name, "scale_mode")) return &t.scale_mode;
+    if (!strcmp(name, "combine_chunks")) return &t.combine_chunks;
+    if (!strcmp(name, "combine_waves")) return &t.combine_waves;
+    if (!strcmp(name, "nontemporal")) return &t.nontemporal;
+    return nullptr;
+}
+
+int mc_ep_world_set_option(mc_ep_world_t* w, const char* name, int value) {
+    MC_ASSERT(w != nullptr && name != nullptr);
+    int* slot = option_slot(w->tuning, name);
+    if (!slot) return fail(MC_EP_ERR_ASSERT, std::string("Failed: unknown option '") + name + "'");
+    *slot = value;
+    return MC_EP_OK;
+}
+
+int mc_ep_world_get_option(const mc_ep_world_t* w, const char* name, int* value) {
+    MC_ASSERT(w != nullptr && name != nullptr && value != nullptr);
+    Tuning t = w->tuning;
+    int* slot = option_slot(t, name);
+    if (!slot) return fail(MC_EP_ERR_ASSERT, std::string("Failed: unknown option '") + name + "'");
+    *value = *slot;
+    return MC_EP_OK;
+}
+
+int mc_ep_world_dispatch(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_t* topk_idx_ptrs,
+                         const int32_t* num_tokens, int hidden, int num_topk, int max_tokens, int num_experts,
+                         int use_fp8, const uint64_t* recv_x_ptrs, const uint64_t* recv_scales_ptrs,
+                         const uint64_t* recv_count_ptrs, const uint64_t* src_info_ptrs,
+                         const uint64_t* layout_range_ptrs, int phases, uint64_t stream_ptr) {
+    MC_ASSERT(w != nullptr);
+    return world_dispatch_impl(w, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, max_tokens, num_experts,
+                               use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
+                               layout_range_ptrs, phases, (hipStream_t)stream_ptr);
+}
+
+int mc_ep_world_combine(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_t* topk_idx_ptrs,
+                        const uint64_t* topk_weights_ptrs, const uint64_t* src_info_ptrs,
+                        const uint64_t* layout_range_ptrs, const uint64_t* active_ranks_ptrs,
+                        const int32_t* num_combined_tokens, int hidden, int num_topk, int max_tokens,
+                        int num_experts, const uint64_t* combined_x_ptrs, int phases, uint64_t stream_ptr) {
+    MC_ASSERT(w != nullptr);
+    return world_combine_impl(w, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
+                              active_ranks_ptrs, num_combined_tokens, hidden, num_topk, max_tokens, num_experts,
+                              combined_x_ptrs, phases, (hipStream_t)stream_ptr);
+}
+
+int mc_ep_buffer_create(mc_ep_world_t* w, int rank, int64_t num_ep_buffer_bytes, int disable_p2p,
+                        mc_ep_buffer_t** out) {
+    MC_ASSERT(w != nullptr && out != nullptr);
+    MC_ASSERT(rank >= 0 && rank < w->R);
+    MC_ASSERT(num_ep_buffer_bytes >= 0);
+    auto* b = new mc_ep_buffer();
+    b->world = w;
+    b->rank = rank;
+    b->num_ep_buffer_bytes = num_ep_buffer_bytes;
+    b->p2p_enabled = !disable_p2p;
+    *out = b;
+    return MC_EP_OK;
+}
+
+int mc_ep_buffer_destroy(mc_ep_buffer_t* b) {
+    delete b;
+    return MC_EP_OK;
+}
+
+int mc_ep_buffer_ibgda_disabled(const mc_ep_buffer_t*) { return 1; }
+int mc_ep_buffer_p2p_enabled(const mc_ep_buffer_t* b) { return b && b->p2p_enabled ? 1 : 0; }
+int mc_ep_buffer_use_fast_path(const mc_ep_buffer_t*) { return 1; }
+int mc_ep_buffer_is_roce(const mc_ep_buffer_t*) { return 0; }
+
+int mc_ep_buffer_dispatch(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_ptr, uint64_t active_ranks_ptr,
+                          int num_tokens, int hidden, int num_topk, int max_tokens, int num_experts,
+                          int timeout_us, int use_fp8, uint64_t recv_x_ptr, uint64_t recv_scales_ptr,
+                          uint64_t recv_count_ptr, uint64_t src_info_ptr, uint64_t layout_range_ptr, int async,
+                          int return_recv_hook, uint64_t compute_stream_ptr, mc_ep_event_t** event_out,
+                          mc_ep_hook_t** hook_out) {
+    MC_ASSERT(b != nullptr && event_out != nullptr && hook_out != nullptr);
+    *event_out = nullptr;
+    *hook_out = nullptr;
+    mc_ep_world* w = b->world;
+    const int num_ranks = w->R;
+    // mooncake_ep_buffer.cpp:202-206
+    MC_ASSERT(num_experts % num_ranks == 0);
+    MC_ASSERT(hidden % 16 == 0 && hidden % 128 == 0);
+    MC_ASSERT(num_tokens <= max_tokens);
+    // :212-214: the reference's communication buffer must hold this shape
+    MC_ASSERT(mc_ep_get_buffer_size_hint(max_tokens, hidden, num_ranks, num_experts) <=
+              (uint64_t)b->num_ep_buffer_bytes);
+    MC_ASSERT(!(async && return_recv_hook));   // :226
+    // :241-251
+    MC_ASSERT(active_ranks_ptr != 0);
+    MC_ASSERT(num_tokens == 0 || (x_ptr != 0 && topk_idx_ptr != 0));
+    MC_ASSERT(recv_x_ptr != 0 && recv_count_ptr != 0);
+    MC_ASSERT(src_info_ptr != 0 && layout_range_ptr != 0);
+    if (use_fp8) {
+        MC_ASSERT(((long long)num_ranks * max_tokens) % 4 == 0);
+        MC_ASSERT(recv_scales_ptr != 0);
+    }
+    MC_ASSERT(num_topk <= kMaxTopK);
+    MC_ASSERT(!w->silent[b->rank]);
+
+    const long long call = w->dispatch_calls[b->rank]++;
+    auto& pr = round_for_call(w, w->dispatch_rounds, w->dispatch_base, call);
+    DispatchPost& p = pr.posts[b->rank];
+    p.present = true;
+    p.x = x_ptr; p.topk_idx = topk_idx_ptr; p.active_ranks = active_ranks_ptr;
+    p.num_tokens = num_tokens; p.hidden = hidden; p.num_topk = num_topk; p.max_tokens = max_tokens;
+    p.num_experts = num_experts; p.timeout_us = timeout_us; p.use_fp8 = use_fp8 ? 1 : 0;
+    p.recv_x = recv_x_ptr; p.recv_scales = recv_scales_ptr; p.recv_count = recv_count_ptr;
+    p.src_info = src_info_ptr; p.layout_range = layout_range_ptr;
+    p.async = async != 0; p.hook = return_recv_hook != 0;
+    p.stream = (hipStream_t)compute_stream_ptr;
+    std::shared_ptr<Round> state = pr.state;
+
+    if (int e = drain_dispatch(w)) return e;
+    if (async) {
+        auto* ev = new mc_ep_event();
+        ev->round = state;
+        *event_out = ev;
+    }
+    if (return_recv_hook) {
+        auto* h = new mc_ep_hook();
+        h->round = state;
+        h->stream = (hipStream_t)compute_stream_ptr;
+        *hook_out = h;
+    }
+    return MC_EP_OK;
+}
+
+int mc_ep_buffer_combine(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_ptr, uint64_t topk_weights_ptr,
+                         uint64_t src_info_ptr, uint64_t layout_range_ptr, uint64_t active_ranks_ptr,
+                         int num_local_experts, int num_combined_tokens, int hidden, int num_topk, int max_tokens,
+                         int num_experts, int timeout_us, int zero_copy, uint64_t combined_x_ptr, int async,
+                         int return_recv_hook, uint64_t compute_stream_ptr, mc_ep_event_t** event_out,
+                         mc_ep_hook_t** hook_out) {
+    MC_ASSERT(b != nullptr && event_out != nullptr && hook_out != nullptr);
+    *event_out = nullptr;
+    *hook_out = nullptr;
+    mc_ep_world* w = b->world;
+    const int num_ranks = w->R;
+    if (zero_copy)
+        return fail(MC_EP_ERR_UNSUPPORTED,
+                    "Mooncake EP zero-copy combine is not supported; pass the expert output tensor to combine() "
+                    "with zero_copy=False");
+    // mooncake_ep_buffer.cpp:351-367
+    MC_ASSERT(num_experts % num_ranks == 0);
+    MC_ASSERT(num_local_experts == num_experts / num_ranks);
+    MC_ASSERT(hidden % 16 == 0 && hidden % 128 == 0);
+    MC_ASSERT(num_combined_tokens <= max_tokens);
+    MC_ASSERT(num_combined_tokens == 0 || (x_ptr != 0 && topk_idx_ptr != 0 && topk_weights_ptr != 0));
+    MC_ASSERT(src_info_ptr != 0 && layout_range_ptr != 0);
+    MC_ASSERT(active_ranks_ptr != 0);
+    MC_ASSERT(num_combined_tokens == 0 || combined_x_ptr != 0);
+    MC_ASSERT(mc_ep_get_buffer_size_hint(max_tokens, hidden, num_ranks, num_experts) <=
+              (uint64_t)b->num_ep_buffer_bytes);   // :370-372
+    MC_ASSERT(!(async && return_recv_hook));       // :384
+    MC_ASSERT(num_topk <= kMaxTopK);
+    MC_ASSERT(!w->silent[b->rank]);
+
+    const long long call = w->combine_calls[b->rank]++;
+    auto& pr = round_for_call(w, w->combine_rounds, w->combine_base, call);
+    CombinePost& p = pr.posts[b->rank];
+    p.present = true;
+    p.x = x_ptr; p.topk_idx = topk_idx_ptr; p.topk_weights = topk_weights_ptr; p.src_info = src_info_ptr;
+    p.layout_range = layout_range_ptr; p.active_ranks = active_ranks_ptr; p.out = combined_x_ptr;
+    p.num_tokens = num_combined_tokens; p.hidden = hidden; p.num_topk = num_topk; p.max_tokens = max_tokens;
+    p.num_experts = num_experts; p.timeout_us = timeout_us;
+    p.async = async != 0; p.hook = return_recv_hook != 0;
+    p.stream = (hipStream_t)compute_stream_ptr;
+    std::shared_ptr<Round> state = pr.state;
+
+    if (int e = drain_combine(w)) return e;
+    if (async) {
+        auto* ev = new mc_ep_event();
+        ev->round = state;
+        *event_out = ev;
+    }
+    if (return_recv_hook) {
+        auto* h = new mc_ep_hook();
+        h->round = state;
+        h->stream = (hipStream_t)compute_stream_ptr;
+        *hook_out = h;
+    }
+    return MC_EP_OK;
+}
+
+int mc_ep_event_create(uint64_t stream_ptr, mc_ep_event_t** out) {
+    MC_ASSERT(out != nullptr);
+    auto ev = std::make_unique<mc_ep_event>();
+    MC_HIP(hipEventCreateWithFlags(&ev->own, hipEventDisableTiming));
+    MC_HIP(hipEventRecord(ev->own, (hipStream_t)stream_ptr));
+    *out = ev.release();
+    return MC_EP_OK;
+}
+
+int mc_ep_event_current_stream_wait(mc_ep_event_t* ev, uint64_t stream_ptr) {
+    MC_ASSERT(ev != nullptr);
+    if (ev->own) {
+        MC_HIP(hipStreamWaitEvent((hipStream_t)stream_ptr, ev->own, 0));
+        return MC_EP_OK;
+    }
+    if (!ev->round || !ev->round->launched) return fail(MC_EP_ERR_PENDING, missing_ranks_message("the call"));
+    MC_HIP(hipStreamWaitEvent((hipStream_t)stream_ptr, ev->round->done, 0));
+    return MC_EP_OK;
+}
+
+int mc_ep_event_synchronize(mc_ep_event_t* ev) {
+    MC_ASSERT(ev != nullptr);
+    if (ev->own) {
+        MC_HIP(hipEventSynchronize(ev->own));
+        return MC_EP_OK;
+    }
+    if (!ev->round || !ev->round->launched) return fail(MC_EP_ERR_PENDING, missing_ranks_message("the call"));
+    MC_HIP(hipEventSynchronize(ev->round->done));
+    return MC_EP_OK;
+}
+
+int mc_ep_event_destroy(mc_ep_event_t* ev) {
+    if (!ev) return MC_EP_OK;
+    if (ev->own) (void)hipEventDestroy(ev->own);
+    delete ev;
+    return MC_EP_OK;
+}
+
+int mc_ep_hook_call(mc_ep_hook_t* h) {
+    MC_ASSERT(h != nullptr);
+    if (!h->round || !h->round->launched) return fail(MC_EP_ERR_PENDING, missing_ranks_message("the call"));
+    MC_HIP(hipStreamWaitEvent(h->stream, h->round->done, 0));
+    return MC_EP_OK;
+}
+
+int mc_ep_hook_destroy(mc_ep_hook_t* h) {
+    delete h;
+    return MC_EP_OK;
+}
+
+int mc_ep_debug_copy(uint64_t dst_ptr, uint64_t src_ptr, uint64_t bytes, uint64_t stream_ptr) {
+    MC_ASSERT(dst_ptr != 0 && src_ptr != 0 && bytes % 16 == 0);
+    MC_HIP(launch_copy((void*)dst_ptr, (const void*)src_ptr, (size_t)bytes, (hipStream_t)stream_ptr));
+    return MC_EP_OK;
+}
+
+}  // extern "C"
