@@ -1,0 +1,98 @@
+"""ctypes loader for libmooncake_ep_hip.so (C ABI: include/mooncake_ep_hip.h).
+
+There is no CPU or PyTorch fallback behind this module: if the HIP library is
+missing, loading raises and every entry point of the package fails with it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_uint64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmooncake_ep_hip.so")
+
+OK, ERR_ASSERT, ERR_HIP, ERR_PENDING, ERR_UNSUPPORTED = 0, 1, 2, 3, 4
+PHASE_LAYOUT, PHASE_DATA, PHASE_ALL = 1, 2, 3
+
+_lib = None
+
+_U64P = POINTER(c_uint64)
+_I32P = POINTER(c_int32)
+_VPP = POINTER(c_void_p)
+
+# name -> (restype, argtypes); one entry per declaration in include/mooncake_ep_hip.h
+SIGNATURES = {
+    "mc_ep_last_error": (c_char_p, []),
+    "mc_ep_get_buffer_size_hint": (c_uint64, [c_int, c_int, c_int, c_int]),
+    "mc_ep_world_create": (c_int, [c_int, _VPP]),
+    "mc_ep_world_destroy": (c_int, [c_void_p]),
+    "mc_ep_world_num_ranks": (c_int, [c_void_p]),
+    "mc_ep_world_set_rank_silent": (c_int, [c_void_p, c_int, c_int]),
+    "mc_ep_world_set_option": (c_int, [c_void_p, c_char_p, c_int]),
+    "mc_ep_world_get_option": (c_int, [c_void_p, c_char_p, POINTER(c_int)]),
+    "mc_ep_world_dispatch": (c_int, [c_void_p, _U64P, _U64P, _I32P, c_int, c_int, c_int, c_int, c_int,
+                                     _U64P, _U64P, _U64P, _U64P, _U64P, c_int, c_uint64]),
+    "mc_ep_world_combine": (c_int, [c_void_p, _U64P, _U64P, _U64P, _U64P, _U64P, _U64P, _I32P, c_int, c_int,
+                                    c_int, c_int, _U64P, c_int, c_uint64]),
+    "mc_ep_buffer_create": (c_int, [c_void_p, c_int, c_int64, c_int, _VPP]),
+    "mc_ep_buffer_destroy": (c_int, [c_void_p]),
+    "mc_ep_buffer_ibgda_disabled": (c_int, [c_void_p]),
+    "mc_ep_buffer_p2p_enabled": (c_int, [c_void_p]),
+    "mc_ep_buffer_use_fast_path": (c_int, [c_void_p]),
+    "mc_ep_buffer_is_roce": (c_int, [c_void_p]),
+    "mc_ep_buffer_dispatch": (c_int, [c_void_p, c_uint64, c_uint64, c_uint64, c_int, c_int, c_int, c_int, c_int,
+                                      c_int, c_int, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_int, c_int,
+                                      c_uint64, _VPP, _VPP]),
+    "mc_ep_buffer_combine": (c_int, [c_void_p, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_uint64, c_int,
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_uint64, c_int, c_int,
+                                     c_uint64, _VPP, _VPP]),
+    "mc_ep_event_create": (c_int, [c_uint64, _VPP]),
+    "mc_ep_event_current_stream_wait": (c_int, [c_void_p, c_uint64]),
+    "mc_ep_event_synchronize": (c_int, [c_void_p]),
+    "mc_ep_event_destroy": (c_int, [c_void_p]),
+    "mc_ep_hook_call": (c_int, [c_void_p]),
+    "mc_ep_hook_destroy": (c_int, [c_void_p]),
+    "mc_ep_debug_copy": (c_int, [c_uint64, c_uint64, c_uint64, c_uint64]),
+}
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is not built; run `make -C {os.path.join(_HERE, 'csrc')}` "
+                "(the dispatch/combine path has no fallback without it)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    msg = lib().mc_ep_last_error()
+    return msg.decode("utf-8", "replace") if msg else ""
+
+
+def check(rc: int) -> None:
+    """Map an MC_EP_ERR_* code to the exception the reference raises: host
+    assertions and HIP failures become RuntimeError (EPException through
+    pybind11), unsupported features NotImplementedError."""
+    if rc == OK:
+        return
+    msg = last_error()
+    if rc == ERR_UNSUPPORTED:
+        raise NotImplementedError(msg)
+    raise RuntimeError(msg)
+
+
+def u64_array(values) -> ctypes.Array:
+    return (c_uint64 * len(values))(*[int(v) for v in values])
+
+
+def i32_array(values) -> ctypes.Array:
+    return (c_int32 * len(values))(*[int(v) for v in values])

@@ -277,7 +277,9 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
 #pragma unroll
     for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(f[j]));
     amax = group_max<8>(amax);
-    const float scale = 448.0f / amax;       // IEEE division: the stored scale is amax / 448, not amax * (1/448)
+    // the arithmetic of CPU PyTorch for `448.0 / amax` (reciprocal, then times
+    // 448) and `amax / 448.0` (true division), both correctly rounded
+    const float scale = (1.0f / amax) * 448.0f;
     const float scale_inv = amax / 448.0f;
     uint32_t o[4];
 #pragma unroll
@@ -342,7 +344,7 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
 #pragma unroll
         for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(f[j]));
         amax = group_max<16>(amax);
-        const float scale = 448.0f / amax;
+        const float scale = (1.0f / amax) * 448.0f;
         scale_inv[p] = amax / 448.0f;
         int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0] * scale, f[1] * scale, 0, false);
         w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2] * scale, f[3] * scale, w0, true);

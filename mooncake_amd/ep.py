@@ -1,0 +1,222 @@
+"""Replacement for the reference's native module `mooncake._ep`
+(mooncake-ep/src/ep_py.cpp:14-46, loaded through mooncake/ep.py:10-17):
+`Buffer`, `EventHandle`, `get_ep_buffer_size_hint`, `MAX_QP_COUNT`, with the
+bound names and argument order of the reference, on top of the C ABI.
+
+One GPU holds the whole expert-parallel world: Buffers created with the same
+`World` (or, by default, with the same `num_ranks` in this process) are the
+logical ranks of one world.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_void_p
+from typing import Callable, Dict, List, Optional, Tuple
+
+from . import _lib
+
+MAX_QP_COUNT = 256   # mooncake_ep_configs.cuh:5
+
+
+def get_ep_buffer_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
+                            num_experts: int) -> int:
+    return int(_lib.lib().mc_ep_get_buffer_size_hint(num_max_dispatch_tokens_per_rank, hidden, num_ranks,
+                                                     num_experts))
+
+
+class World:
+    """R logical EP ranks resident in the current device's HBM."""
+
+    def __init__(self, num_ranks: int):
+        handle = c_void_p()
+        _lib.check(_lib.lib().mc_ep_world_create(int(num_ranks), ctypes.byref(handle)))
+        self._h = handle
+        self.num_ranks = int(num_ranks)
+
+    def close(self) -> None:
+        if self._h:
+            _lib.lib().mc_ep_world_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_rank_silent(self, rank: int, silent: bool = True) -> None:
+        """The rank stops calling dispatch/combine (a failed process)."""
+        _lib.check(_lib.lib().mc_ep_world_set_rank_silent(self._h, int(rank), int(bool(silent))))
+
+    def set_option(self, name: str, value: int) -> None:
+        _lib.check(_lib.lib().mc_ep_world_set_option(self._h, name.encode(), int(value)))
+
+    def get_option(self, name: str) -> int:
+        out = ctypes.c_int()
+        _lib.check(_lib.lib().mc_ep_world_get_option(self._h, name.encode(), ctypes.byref(out)))
+        return out.value
+
+    # whole-world calls: every rank's tensors in one launch sequence
+    def dispatch(self, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
+                 num_experts, use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
+                 layout_range_ptrs, stream_ptr: int, phases: int = _lib.PHASE_ALL) -> None:
+        u = _lib.u64_array
+        scales = u(recv_scales_ptrs) if recv_scales_ptrs is not None else None
+        _lib.check(_lib.lib().mc_ep_world_dispatch(
+            self._h, u(x_ptrs), u(topk_idx_ptrs), _lib.i32_array(num_tokens), hidden, num_topk,
+            num_max_dispatch_tokens_per_rank, num_experts, int(bool(use_fp8)), u(recv_x_ptrs), scales,
+            u(recv_count_ptrs), u(src_info_ptrs), u(layout_range_ptrs), phases, stream_ptr))
+
+    def combine(self, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
+                active_ranks_ptrs, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
+                num_experts, combined_x_ptrs, stream_ptr: int, phases: int = _lib.PHASE_ALL) -> None:
+        u = _lib.u64_array
+        _lib.check(_lib.lib().mc_ep_world_combine(
+            self._h, u(x_ptrs), u(topk_idx_ptrs), u(topk_weights_ptrs), u(src_info_ptrs), u(layout_range_ptrs),
+            u(active_ranks_ptrs), _lib.i32_array(num_combined_tokens), hidden, num_topk,
+            num_max_dispatch_tokens_per_rank, num_experts, u(combined_x_ptrs), phases, stream_ptr))
+
+
+_default_worlds: Dict[int, World] = {}
+
+
+def default_world(num_ranks: int) -> World:
+    """The process-wide world that Buffers of `num_ranks` ranks join unless told otherwise."""
+    w = _default_worlds.get(num_ranks)
+    if w is None or w._h is None:
+        w = World(num_ranks)
+        _default_worlds[num_ranks] = w
+    return w
+
+
+class EventHandle:
+    """mooncake_ep_event.h:9-42."""
+
+    def __init__(self, stream_ptr: int = 0, _handle: Optional[c_void_p] = None):
+        if _handle is not None:
+            self._h = _handle
+        else:
+            handle = c_void_p()
+            _lib.check(_lib.lib().mc_ep_event_create(int(stream_ptr), ctypes.byref(handle)))
+            self._h = handle
+
+    def current_stream_wait(self, stream_ptr: int) -> None:
+        _lib.check(_lib.lib().mc_ep_event_current_stream_wait(self._h, int(stream_ptr)))
+
+    def synchronize(self) -> None:
+        _lib.check(_lib.lib().mc_ep_event_synchronize(self._h))
+
+    def __del__(self):
+        try:
+            if self._h:
+                _lib.lib().mc_ep_event_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class _RecvHook:
+    def __init__(self, handle: c_void_p):
+        self._h = handle
+
+    def __call__(self) -> None:
+        _lib.check(_lib.lib().mc_ep_hook_call(self._h))
+
+    def __del__(self):
+        try:
+            if self._h:
+                _lib.lib().mc_ep_hook_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class Buffer:
+    """One logical rank's MooncakeEpBuffer (ep_py.cpp:26-46)."""
+
+    def __init__(self, rank: int, num_ranks: int, num_ep_buffer_bytes: int, disable_p2p: bool = False,
+                 world: Optional[World] = None):
+        self.world = world if world is not None else default_world(num_ranks)
+        if self.world.num_ranks != num_ranks:
+            raise RuntimeError(f"world has {self.world.num_ranks} ranks, Buffer asked for {num_ranks}")
+        handle = c_void_p()
+        _lib.check(_lib.lib().mc_ep_buffer_create(self.world._h, int(rank), int(num_ep_buffer_bytes),
+                                                  int(bool(disable_p2p)), ctypes.byref(handle)))
+        self._h = handle
+        self.rank = int(rank)
+        self.num_ranks = int(num_ranks)
+
+    def __del__(self):
+        try:
+            if self._h:
+                _lib.lib().mc_ep_buffer_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+    # --- transport introspection: one address space, no NIC ---------------
+    def ibgda_disabled(self) -> bool:
+        return bool(_lib.lib().mc_ep_buffer_ibgda_disabled(self._h))
+
+    def p2p_enabled(self) -> bool:
+        return bool(_lib.lib().mc_ep_buffer_p2p_enabled(self._h))
+
+    def use_fast_path(self) -> bool:
+        return bool(_lib.lib().mc_ep_buffer_use_fast_path(self._h))
+
+    def is_roce(self) -> bool:
+        return bool(_lib.lib().mc_ep_buffer_is_roce(self._h))
+
+    def update_local_qpns(self) -> None:
+        return None
+
+    def sync_ibgda_peers(self, remote_addrs, remote_keys, peer_qpns, peer_lids, subnet_prefixes, interface_ids,
+                         active_ranks_mask) -> None:
+        return None
+
+    def get_mr_info(self) -> Tuple[int, int]:
+        return (0, 0)
+
+    def get_gid(self) -> Tuple[int, int]:
+        return (0, 0)
+
+    def get_local_qpns(self) -> List[int]:
+        return []
+
+    def get_local_lids(self) -> List[int]:
+        return []
+
+    def get_ipc_handle(self) -> List[int]:
+        return []
+
+    def sync_nvlink_ipc_handles(self, remote_handles, active_ranks_mask) -> None:
+        return None
+
+    # --- the two hot calls ------------------------------------------------
+    def dispatch(self, x_ptr: int, topk_idx_ptr: int, active_ranks_ptr: int, num_tokens: int, hidden: int,
+                 num_topk: int, num_max_dispatch_tokens_per_rank: int, num_experts: int, timeout_us: int,
+                 use_fp8: bool, packed_recv_x_ptr: int, packed_recv_x_scales_ptr: int, packed_recv_count_ptr: int,
+                 packed_recv_src_info_ptr: int, packed_recv_layout_range_ptr: int, async_: bool,
+                 return_recv_hook: bool, compute_stream_ptr: int
+                 ) -> Tuple[Optional[EventHandle], Optional[Callable[[], None]]]:
+        ev, hook = c_void_p(), c_void_p()
+        _lib.check(_lib.lib().mc_ep_buffer_dispatch(
+            self._h, x_ptr, topk_idx_ptr, active_ranks_ptr, num_tokens, hidden, num_topk,
+            num_max_dispatch_tokens_per_rank, num_experts, timeout_us, int(bool(use_fp8)), packed_recv_x_ptr,
+            packed_recv_x_scales_ptr, packed_recv_count_ptr, packed_recv_src_info_ptr,
+            packed_recv_layout_range_ptr, int(bool(async_)), int(bool(return_recv_hook)), compute_stream_ptr,
+            ctypes.byref(ev), ctypes.byref(hook)))
+        return (EventHandle(_handle=ev) if ev else None, _RecvHook(hook) if hook else None)
+
+    def combine(self, x_ptr: int, topk_idx_ptr: int, topk_weights_ptr: int, src_info_ptr: int,
+                layout_range_ptr: int, active_ranks_ptr: int, num_local_experts: int, num_combined_tokens: int,
+                hidden: int, num_topk: int, num_max_dispatch_tokens_per_rank: int, num_experts: int,
+                timeout_us: int, zero_copy: bool, combined_x_ptr: int, async_: bool, return_recv_hook: bool,
+                compute_stream_ptr: int) -> Tuple[Optional[EventHandle], Optional[Callable[[], None]]]:
+        ev, hook = c_void_p(), c_void_p()
+        _lib.check(_lib.lib().mc_ep_buffer_combine(
+            self._h, x_ptr, topk_idx_ptr, topk_weights_ptr, src_info_ptr, layout_range_ptr, active_ranks_ptr,
+            num_local_experts, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
+            num_experts, timeout_us, int(bool(zero_copy)), combined_x_ptr, int(bool(async_)),
+            int(bool(return_recv_hook)), compute_stream_ptr, ctypes.byref(ev), ctypes.byref(hook)))
+        return (EventHandle(_handle=ev) if ev else None, _RecvHook(hook) if hook else None)

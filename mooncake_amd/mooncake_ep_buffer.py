@@ -1,0 +1,210 @@
+"""Python `Buffer` for the low-latency dispatch/combine path with the
+signature, checks and return shapes of the reference wrapper
+(mooncake-wheel/mooncake/mooncake_ep_buffer.py:92-119, :360-535, :538-681),
+running on the HIP library for one MI355X.
+
+The expert-parallel world is a set of logical ranks in one process: a
+`LogicalGroup` stands in for the torch process group (`rank()`, `size()`),
+and dispatch/combine are collectives over the group's ranks - the kernels for
+all ranks are launched by the call that completes the round, so outputs are
+valid (in stream order) once every live rank has made its call.
+"""
+from __future__ import annotations
+
+from typing import Any, Callable, Optional, Tuple, Union
+
+import torch
+
+from . import ep
+
+_ZERO_COPY_COMBINE_UNSUPPORTED = (
+    "Mooncake EP zero-copy combine is not supported; pass the expert output "
+    "tensor to combine() with zero_copy=False"
+)
+
+
+def _native_current_stream_ptr() -> int:
+    return int(torch.cuda.current_stream().cuda_stream)
+
+
+class LogicalGroup:
+    """Stands in for `dist.ProcessGroup`: one logical rank of an `ep.World`."""
+
+    def __init__(self, world: ep.World, rank: int):
+        assert 0 <= rank < world.num_ranks
+        self.world = world
+        self._rank = int(rank)
+
+    def rank(self) -> int:
+        return self._rank
+
+    def size(self) -> int:
+        return self.world.num_ranks
+
+    @staticmethod
+    def make_world(num_ranks: int):
+        """A fresh world and its R groups."""
+        world = ep.World(num_ranks)
+        return world, [LogicalGroup(world, r) for r in range(num_ranks)]
+
+
+class EventOverlap:
+    """Event wrapper with the `with` protocol (reference :34-89)."""
+
+    def __init__(self, event: Optional[ep.EventHandle] = None,
+                 extra_tensors: Optional[Tuple[torch.Tensor, ...]] = None) -> None:
+        self.event = event
+        # keeps inputs/outputs alive until the event has been waited on
+        self.extra_tensors = extra_tensors
+
+    def current_stream_wait(self) -> None:
+        assert self.event is not None
+        self.event.current_stream_wait(_native_current_stream_ptr())
+
+    def __enter__(self) -> Any:
+        return self
+
+    def __exit__(self, exc_type: Any, exc_val: Any, exc_tb: Any) -> None:
+        if self.event is not None:
+            self.event.current_stream_wait(_native_current_stream_ptr())
+
+
+class Buffer:
+    def __init__(self, group, num_ep_buffer_bytes: int = 0, disable_p2p: bool = False):
+        self.rank = group.rank()
+        self.group_size = group.size()
+        self.group = group
+        self.num_ep_buffer_bytes = num_ep_buffer_bytes
+        self.backend = self.group
+        world = getattr(group, "world", None)
+        self.runtime = ep.Buffer(self.rank, self.group_size, num_ep_buffer_bytes, disable_p2p, world=world)
+        # there is no slow path here: the HIP kernels are the only implementation
+        self._use_fallback = False
+        self.connect()
+
+    def connect(self, active_ranks=None) -> None:
+        """Peer exchange of the reference (:185-304) has nothing to do when
+        every rank lives in the same address space."""
+        if not self.runtime.use_fast_path():
+            raise RuntimeError("mooncake_amd has no fallback path")
+
+    def update_ep_member(self) -> None:
+        self.connect(True)
+
+    @staticmethod
+    def get_ep_buffer_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
+                                num_experts: int) -> int:
+        return ep.get_ep_buffer_size_hint(num_max_dispatch_tokens_per_rank, hidden, num_ranks, num_experts)
+
+    def _default_active_ranks(self, device: torch.device) -> torch.Tensor:
+        return torch.ones((self.group_size,), dtype=torch.int32, device=device)
+
+    # noinspection PyTypeChecker
+    def dispatch(self, x: torch.Tensor, topk_idx: torch.Tensor, active_ranks: Optional[torch.Tensor],
+                 num_max_dispatch_tokens_per_rank: int, num_experts: int, timeout_us: int,
+                 use_fp8: Optional[bool] = None, async_finish: bool = False, return_recv_hook: bool = False,
+                 ) -> Tuple[Union[Tuple[torch.Tensor, torch.Tensor], torch.Tensor], torch.Tensor, Tuple,
+                            EventOverlap, Callable]:
+        assert x.dim() == 2 and x.is_contiguous()
+        assert x.dtype == torch.bfloat16
+        assert topk_idx.dim() == 2 and topk_idx.is_contiguous()
+        assert topk_idx.dtype == torch.int64
+        assert x.size(0) == topk_idx.size(0)
+        assert x.size(0) <= num_max_dispatch_tokens_per_rank
+        assert x.size(1) % 16 == 0 and x.size(1) % 128 == 0
+        assert num_experts % self.group_size == 0
+        if active_ranks is None:
+            active_ranks = self._default_active_ranks(x.device)
+        else:
+            assert active_ranks.dim() == 1 and active_ranks.is_contiguous()
+            assert active_ranks.dtype == torch.int32
+            if active_ranks.numel() != self.group_size:
+                active_ranks = self._default_active_ranks(x.device)
+        if use_fp8 is None:
+            use_fp8 = True
+
+        num_local_experts = num_experts // self.group_size
+        rm = self.group_size * num_max_dispatch_tokens_per_rank
+        hidden = x.size(1)
+        # outputs are not cleared: rows at and beyond packed_recv_count stay unwritten
+        packed_recv_x = torch.empty((num_local_experts, rm, hidden),
+                                    dtype=torch.float8_e4m3fn if use_fp8 else torch.bfloat16, device=x.device)
+        packed_recv_count = torch.empty((num_local_experts,), dtype=torch.int32, device=x.device)
+        packed_recv_src_info = torch.empty((num_local_experts, rm), dtype=torch.int32, device=x.device)
+        packed_recv_layout_range = torch.empty((num_local_experts, self.group_size), dtype=torch.int64,
+                                               device=x.device)
+        packed_recv_x_scales = None
+        if use_fp8:
+            assert rm % 4 == 0
+            # column-major per expert: [L, H/128, R*max] storage viewed as [L, R*max, H/128]
+            packed_recv_x_scales = torch.empty((num_local_experts, hidden // 128, rm), dtype=torch.float32,
+                                               device=x.device).transpose(1, 2)
+        event, hook = self.runtime.dispatch(
+            x.data_ptr(), topk_idx.data_ptr(), active_ranks.data_ptr(), x.size(0), hidden, topk_idx.size(1),
+            num_max_dispatch_tokens_per_rank, num_experts, timeout_us, use_fp8, packed_recv_x.data_ptr(),
+            0 if packed_recv_x_scales is None else packed_recv_x_scales.data_ptr(), packed_recv_count.data_ptr(),
+            packed_recv_src_info.data_ptr(), packed_recv_layout_range.data_ptr(), async_finish, return_recv_hook,
+            _native_current_stream_ptr())
+        handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, hidden,
+                  num_experts)
+        tensors_to_record = (x, topk_idx, active_ranks, packed_recv_x, packed_recv_x_scales, packed_recv_count,
+                             packed_recv_src_info, packed_recv_layout_range)
+        # inputs of a deferred collective must outlive this call: the round
+        # may be launched by a later rank's call
+        self._pending_dispatch_refs = tensors_to_record
+        return ((packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x, packed_recv_count, handle,
+                EventOverlap(event, tensors_to_record if async_finish else None), hook)
+
+    # noinspection PyTypeChecker
+    def combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
+                active_ranks: Optional[torch.Tensor], timeout_us: int, handle: tuple, zero_copy: bool = False,
+                async_finish: bool = False, return_recv_hook: bool = False, out: Optional[torch.Tensor] = None,
+                ) -> Tuple[torch.Tensor, EventOverlap, Callable]:
+        if zero_copy:
+            raise NotImplementedError(_ZERO_COPY_COMBINE_UNSUPPORTED)
+        assert x.dim() == 3 and x.is_contiguous()
+        assert x.dtype == torch.bfloat16
+        assert topk_idx.dim() == 2 and topk_idx.is_contiguous()
+        assert topk_idx.dtype == torch.int64
+        assert topk_weights.dim() == 2 and topk_weights.is_contiguous()
+        assert topk_weights.dtype == torch.float32
+        if active_ranks is None:
+            active_ranks = self._default_active_ranks(x.device)
+        else:
+            assert active_ranks.dim() == 1 and active_ranks.is_contiguous()
+            assert active_ranks.dtype == torch.int32
+            if active_ranks.numel() != self.group_size:
+                active_ranks = self._default_active_ranks(x.device)
+        src_info, layout_range, num_max_dispatch_tokens_per_rank, hidden, num_experts = handle
+        assert x.size(0) == num_experts // self.group_size
+        assert x.size(1) == self.group_size * num_max_dispatch_tokens_per_rank
+        assert x.size(2) == hidden
+        assert x.size(2) % 16 == 0 and x.size(2) % 128 == 0
+        assert topk_idx.size() == topk_weights.size()
+        assert topk_weights.size(0) <= num_max_dispatch_tokens_per_rank
+        assert src_info.dim() == 2 and src_info.is_contiguous()
+        assert src_info.dtype == torch.int32
+        assert src_info.size(0) == x.size(0)
+        assert layout_range.dim() == 2 and layout_range.is_contiguous()
+        assert layout_range.dtype == torch.int64
+        assert layout_range.size(0) == num_experts // self.group_size
+        assert layout_range.size(1) == self.group_size
+        if out is not None:
+            assert out.dim() == 2 and out.is_contiguous()
+            assert out.size(0) == topk_weights.size(0)
+            assert out.size(1) == hidden
+            assert out.dtype == x.dtype
+            combined_x = out
+        else:
+            combined_x = torch.empty((topk_weights.size(0), hidden), dtype=x.dtype, device=x.device)
+        event, hook = self.runtime.combine(
+            x.data_ptr(), topk_idx.data_ptr(), topk_weights.data_ptr(), src_info.data_ptr(),
+            layout_range.data_ptr(), active_ranks.data_ptr(), x.size(0), topk_weights.size(0), hidden,
+            topk_weights.size(1), num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy,
+            combined_x.data_ptr(), async_finish, return_recv_hook, _native_current_stream_ptr())
+        tensors_to_record = (x, topk_idx, topk_weights, active_ranks, src_info, layout_range, combined_x)
+        self._pending_combine_refs = tensors_to_record
+        return combined_x, EventOverlap(event, tensors_to_record if async_finish else None), hook
+
+    def get_next_combine_buffer(self, handle: object):
+        raise NotImplementedError(_ZERO_COPY_COMBINE_UNSUPPORTED)

@@ -124,15 +124,20 @@ ORACLE_API void oracle_f32_to_bf16(const float* in, uint16_t* out, int64_t n) {
 /* per-128 quantisation of one row                                           */
 /* ------------------------------------------------------------------------ */
 
-/* PY:694-703 == TU:42-47 (amax clamp 1e-4, payload f32(x) * (448 / amax) cast
- * to e4m3fn, stored scale amax / 448) with the kernel's group size and amax
- * floor (K:183-186, K:243-252).  NaN elements do not raise amax (fmaxf, K:247);
- * they encode as fp8 NaN themselves. */
+/* PY:694-703 == TU:42-47 (amax clamp 1e-4, payload f32(x) * (448.0 / amax)
+ * cast to e4m3fn, stored scale amax / 448.0) with the kernel's group size and
+ * amax floor (K:183-186, K:243-252).  The arithmetic is the one CPU PyTorch
+ * performs for those two expressions: `448.0 / tensor` is Tensor.__rtruediv__,
+ * i.e. reciprocal() * 448.0 - two roundings, different from the IEEE quotient
+ * 448 / amax (which K:252 computes) in about a quarter of all groups - while
+ * `tensor / 448.0` is a true IEEE division (K:252 multiplies by 1/448
+ * instead).  tests/test_oracle_fp8.py pins both against torch itself.
+ * NaN elements do not raise amax (fmaxf, K:247); they encode as fp8 NaN. */
 static void quantise_row(const uint16_t* x, int H, uint8_t* q, float* scales, int64_t scale_stride) {
     for (int g = 0; g < H / 128; ++g) {
         float amax = 1e-4f;
         for (int j = 0; j < 128; ++j) amax = fmaxf(amax, fabsf(bf16_to_f32(x[g * 128 + j])));
-        float scale = 448.0f / amax;
+        float scale = (1.0f / amax) * 448.0f;
         float scale_inv = amax / 448.0f;
         for (int j = 0; j < 128; ++j) q[g * 128 + j] = f32_to_e4m3fn(bf16_to_f32(x[g * 128 + j]) * scale);
         scales[(int64_t)g * scale_stride] = scale_inv;

@@ -105,11 +105,12 @@ def layout(topk_idx: torch.Tensor, num_tokens: Sequence[int], max_tokens: int, n
 
 def dispatch(x: torch.Tensor, topk_idx: torch.Tensor, num_tokens: Sequence[int], max_tokens: int,
              num_experts: int, use_fp8: bool, src_present: Optional[Sequence[int]] = None,
-             poison: int = -7) -> Dict[str, torch.Tensor]:
+             poison: Optional[int] = -7) -> Dict[str, torch.Tensor]:
     """Whole-world dispatch.  x bf16 [R, Tmax, H], topk_idx int64 [R, Tmax, K].
 
     Returns recv_x ([R,L,RM,H] float8_e4m3fn or bf16; unwritten rows keep the
-    byte pattern 0xA5), scales (logical [R,L,RM,H/128] view of a physical
+    byte pattern 0xA5, or are uninitialised - and never touched, so that large
+    worlds cost only their valid rows - when poison is None), scales (logical [R,L,RM,H/128] view of a physical
     [R,L,H/128,RM] tensor, or None), recv_count, src_info, layout_range, slot_map.
     """
     assert x.dtype == torch.bfloat16 and x.dim() == 3
@@ -121,17 +122,20 @@ def dispatch(x: torch.Tensor, topk_idx: torch.Tensor, num_tokens: Sequence[int],
     L = E // R
     RM = R * max_tokens
     G = H // 128
+    def _new(shape, dtype, fill):
+        return torch.empty(shape, dtype=dtype) if poison is None else torch.full(shape, fill, dtype=dtype)
+
     if use_fp8:
-        recv_x = torch.full((R, L, RM, H), 0xA5, dtype=torch.uint8)
-        scales_phys = torch.full((R, L, G, RM), float("nan"), dtype=torch.float32)
+        recv_x = _new((R, L, RM, H), torch.uint8, 0xA5)
+        scales_phys = _new((R, L, G, RM), torch.float32, float("nan"))
     else:
-        recv_x = torch.full((R, L, RM, H), 0xA5A5 - 65536, dtype=torch.int16)
+        recv_x = _new((R, L, RM, H), torch.int16, 0xA5A5 - 65536)
         scales_phys = None
     out = {
-        "recv_count": torch.full((R, L), poison, dtype=torch.int32),
-        "layout_range": torch.full((R, L, R), poison, dtype=torch.int64),
-        "src_info": torch.full((R, L, RM), poison, dtype=torch.int32),
-        "slot_map": torch.full((R, Tmax, K), poison, dtype=torch.int32),
+        "recv_count": _new((R, L), torch.int32, poison),
+        "layout_range": _new((R, L, R), torch.int64, poison),
+        "src_info": _new((R, L, RM), torch.int32, poison),
+        "slot_map": _new((R, Tmax, K), torch.int32, poison),
     }
     nt = _i32(num_tokens)
     sp = None if src_present is None else _i32(src_present)

@@ -1,0 +1,184 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle
+on the same seeded inputs.  Bit-exact for counts, ranges, source indices, fp8
+payload and scales, bf16 payload; combine bit-exact against the oracle's fused
+fp32 chain and within one bf16 ulp of a float64 sum."""
+import pytest
+import torch
+
+from mooncake_amd.workloads import CONFIGS, EPConfig, generate, shrink
+from tests import ref_checks as rc
+from tests.gpu_util import announce, compare_dispatch, run_dispatch
+
+pytestmark = pytest.mark.gpu
+
+SMALL = [
+    EPConfig("tiny_bf16", 2, 4, 128, 4, 2, False),
+    EPConfig("tiny_fp8", 2, 4, 128, 4, 2, True),
+    EPConfig("odd_hidden_fp8", 4, 24, 2560, 16, 3, True),            # 2.5 slabs of 1024
+    EPConfig("odd_hidden_bf16", 4, 24, 2560, 16, 3, False),
+    EPConfig("k11", 4, 40, 2048, 32, 11, True),                      # the reference's top-k cap
+    EPConfig("k16_bf16", 2, 20, 1024, 32, 16, False),
+    EPConfig("one_rank", 1, 36, 1024, 6, 2, True),                   # group_size == 1
+    EPConfig("masked", 8, 64, 1024, 8, 2, False, masked_fraction=0.3),
+    EPConfig("zipf_outliers", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05),
+    shrink(CONFIGS["cpu_check"]),                                    # the contract's CPU-reference case, full size
+]
+
+
+def ragged(cfg, on):
+    if not on:
+        return None
+    return [max(0, cfg.tokens_per_rank - (r * 5) % (cfg.tokens_per_rank + 1)) for r in range(cfg.num_ranks)]
+
+
+@pytest.mark.parametrize("cfg", SMALL, ids=[c.name for c in SMALL])
+@pytest.mark.parametrize("is_ragged", [False, True], ids=["full", "ragged"])
+def test_dispatch_matches_oracle(gpu_device, oracle, cfg, is_ragged):
+    nt = ragged(cfg, is_ragged)
+    announce(f"dispatch {cfg} ragged={nt}")
+    data = generate(cfg, seed=0)
+    h = run_dispatch(cfg, data, num_tokens=nt, poison=True)
+    ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, cfg.use_fp8)
+    compare_dispatch(h, ref, check_poison=True)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("nontemporal", [0, 3])
+def test_fp8_pack_variants_match_oracle(gpu_device, oracle, variant, nontemporal):
+    cfg = EPConfig("variants", 4, 24, 2560, 16, 3, True)
+    announce(f"pack variant={variant} nontemporal={nontemporal}")
+    data = generate(cfg, seed=1)
+    h = run_dispatch(cfg, data, poison=True, options={"pack_variant": variant, "nontemporal": nontemporal})
+    ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, True)
+    compare_dispatch(h, ref, check_poison=True)
+
+
+def test_fp8_every_bf16_value(gpu_device, oracle):
+    """All finite bf16 bit patterns through the quantiser, in shuffled groups
+    (mixed magnitudes) and in sorted groups (tiny amax, subnormal payloads)."""
+    bits = torch.arange(0, 65536, dtype=torch.int32)
+    vals = (bits << 16).view(torch.float32)
+    vals = vals[torch.isfinite(vals)]
+    g = torch.Generator().manual_seed(11)
+    H = 1024
+    pad = (-vals.numel()) % H
+    shuffled = torch.cat([vals[torch.randperm(vals.numel(), generator=g)], torch.zeros(pad)])
+    ordered = torch.cat([vals.sort().values, torch.zeros(pad)])
+    rows = torch.cat([shuffled, ordered]).view(-1, H).to(torch.bfloat16)       # 128 rows
+    T = rows.size(0)
+    cfg = EPConfig("all_bf16", 1, T, H, 2, 1, True)
+    announce(f"every bf16 value: {T} rows of {H}")
+    data = {"x": rows.unsqueeze(0).contiguous(),
+            "topk_idx": (torch.arange(T) % 2).view(1, T, 1).to(torch.int64),
+            "topk_weights": torch.ones(1, T, 1)}
+    h = run_dispatch(cfg, data, poison=True)
+    ref = oracle.dispatch(data["x"], data["topk_idx"], [T], T, 2, True)
+    compare_dispatch(h, ref, check_poison=True)
+    # and against the reference's formula executed by torch
+    q_ref, s_ref = rc.reference_fp8_cast(rows)
+    got = h.recv_x.cpu()[0]                                                    # [2, T, H]
+    si = h.src_info.cpu()[0]
+    for e in range(2):
+        n = int(h.recv_count[0, e])
+        assert torch.equal(got[e, :n], q_ref.view(torch.uint8)[si[e, :n].long()])
+        assert torch.equal(h.recv_scales()[0, e, :n].cpu().contiguous().view(torch.int32),
+                           s_ref[si[e, :n].long()].contiguous().view(torch.int32))
+
+
+def test_fp8_inf_and_nan_inputs(gpu_device, oracle):
+    H, T = 1024, 8
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    x[1, 5] = float("inf")
+    x[2, 700] = float("-inf")
+    x[3, 130] = float("nan")
+    cfg = EPConfig("nonfinite", 1, T, H, 1, 1, True)
+    announce("fp8 inf / nan inputs")
+    data = {"x": x.unsqueeze(0).contiguous(), "topk_idx": torch.zeros(1, T, 1, dtype=torch.int64),
+            "topk_weights": torch.ones(1, T, 1)}
+    h = run_dispatch(cfg, data, poison=True)
+    ref = oracle.dispatch(data["x"], data["topk_idx"], [T], T, 1, True)
+    got, want = h.recv_x.cpu()[0, 0, :T], ref["recv_x"].view(torch.uint8)[0, 0, :T]
+    # NaN payload bytes: both must be a NaN encoding (0x7F / 0xFF); everything else bit-exact
+    nan_w = (want & 0x7F) == 0x7F
+    assert torch.equal((got & 0x7F) == 0x7F, nan_w)
+    assert torch.equal(got[~nan_w], want[~nan_w])
+    assert torch.equal(h.recv_scales()[0, 0, :T].cpu().contiguous().view(torch.int32),
+                       ref["scales"][0, 0, :T].contiguous().view(torch.int32))
+
+
+COMBINE_CASES = [
+    EPConfig("tiny_c", 2, 4, 128, 4, 2, False),
+    EPConfig("odd_hidden_c", 4, 24, 2560, 16, 3, False),
+    EPConfig("k11_c", 4, 40, 2048, 32, 11, False),
+    EPConfig("k16_c", 2, 20, 1024, 32, 16, False),
+    EPConfig("masked_c", 8, 64, 1024, 8, 2, False, masked_fraction=0.3),
+    EPConfig("fp8_c", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05),
+    shrink(CONFIGS["cpu_check"]),
+]
+
+
+@pytest.mark.parametrize("cfg", COMBINE_CASES, ids=[c.name for c in COMBINE_CASES])
+@pytest.mark.parametrize("is_ragged", [False, True], ids=["full", "ragged"])
+@pytest.mark.parametrize("chunks", [1, 2])
+def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks):
+    nt = ragged(cfg, is_ragged)
+    announce(f"combine {cfg} ragged={nt} chunks={chunks}")
+    data = generate(cfg, seed=3)
+    h = run_dispatch(cfg, data, num_tokens=nt, poison=False, options={"combine_chunks": chunks})
+    factor = torch.arange(cfg.num_experts).float() * 0.1 + 1.0
+    h.alloc_combine_io()
+    h.expert_out.fill_(float("nan"))                       # rows outside the handle must never be read
+    h.fill_expert_out_from_recv(factor)
+    # keep NaN in every padding row
+    RM = cfg.num_ranks * cfg.max_tokens
+    pad = torch.arange(RM, device=h.recv_count.device).view(1, 1, RM) >= h.recv_count.unsqueeze(-1)
+    h.expert_out[pad] = float("nan")
+    h.combined.fill_(7.0)
+    h.combine()
+    torch.cuda.synchronize()
+    eo = h.expert_out.cpu()
+    ref_d = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, cfg.use_fp8)
+    want = oracle.combine(eo, data["topk_idx"], data["topk_weights"], ref_d["src_info"], ref_d["layout_range"],
+                          h.num_tokens, cfg.max_tokens, cfg.num_experts, use_fma=True)
+    got = h.combined.cpu()
+    exact = rc.combine_fp64(torch.nan_to_num(eo.float()).to(torch.bfloat16), data["topk_idx"], data["topk_weights"],
+                            ref_d["slot_map"], h.num_tokens, cfg.max_tokens, cfg.num_experts)
+    for r, n in enumerate(h.num_tokens):
+        assert torch.equal(got[r, :n].view(torch.int16), want[r, :n].view(torch.int16)), f"rank {r}"
+        assert bool(rc.within_one_ulp_of(got[r, :n], exact[r, :n]).all()), f"rank {r} vs float64"
+        assert bool((got[r, n:] == 7.0).all()), "rows beyond num_tokens written"
+
+
+def test_combine_skips_inactive_ranks(gpu_device, oracle):
+    cfg = EPConfig("inactive", 4, 16, 1024, 16, 4, False)
+    announce("combine with an inactive rank")
+    data = generate(cfg, seed=4)
+    h = run_dispatch(cfg, data, poison=False)
+    h.alloc_combine_io()
+    h.fill_expert_out_from_recv(torch.arange(16).float() * 0.1 + 1.0)
+    h.active_ranks[:, 2] = 0
+    h.active_ranks[3, 1] = 0                              # views differ per rank
+    h.combine()
+    torch.cuda.synchronize()
+    want = oracle.combine(h.expert_out.cpu(), data["topk_idx"], data["topk_weights"], h.src_info.cpu(),
+                          h.layout_range.cpu(), h.num_tokens, cfg.max_tokens, cfg.num_experts,
+                          active=h.active_ranks.cpu())
+    assert torch.equal(h.combined.cpu().view(torch.int16), want.view(torch.int16))
+
+
+def test_dispatch_with_silent_rank(gpu_device, oracle):
+    cfg = EPConfig("silent", 4, 16, 1024, 16, 4, True)
+    announce("dispatch with a silent rank")
+    data = generate(cfg, seed=5)
+    present = [1, 1, 0, 1]
+    h = run_dispatch(cfg, data, poison=True, present=present)
+    ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, True,
+                          src_present=present)
+    # the silent rank's own outputs are never written
+    assert bool((h.recv_count[2] == -7).all()) and bool((h.src_info[2] == -7).all())
+    for k in ("recv_count", "layout_range", "src_info"):
+        ref[k][2] = -7
+    h.recv_count[2] = 0
+    ref["recv_count"][2] = 0
+    compare_dispatch(h, ref, check_poison=False)
