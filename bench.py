@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the dispatch + combine hot path on one MI355X.
+
+A step is one whole-world dispatch followed by one whole-world combine of the
+DeepSeek-V3 decode configuration (32 logical ranks x 128 tokens, hidden 7168,
+256 experts, top-8, fp8 dispatch, bf16 combine), all ranks' tensors resident
+in HBM before the timed region.  Prints one JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME]
+                    [--no-cpu-baseline] [--opt name=value ...]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
+METRIC = "dispatch+combine µs & HBM GB/s (% peak), DSV3 decode 128 tok top-8 fp8"
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="dsv3_decode")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget for the cpu_baseline sample")
+    ap.add_argument("--kernel-iters", type=int, default=30, help="timed launches per kernel for the roofline figures")
+    ap.add_argument("--opt", action="append", default=[], help="library tuning option, name=value")
+    return ap.parse_args()
+
+
+def time_kernel(fn, iters, between=None):
+    """Average device time of one launch of `fn`: events on the launch stream
+    around each launch, the stream idle before the start event (so the event
+    pair brackets this launch only); `between` runs untimed before each sample
+    to put the caches in the state the real step leaves them in.  The first
+    sample is dropped."""
+    import torch
+    ms = []
+    for _ in range(iters + 1):
+        if between is not None:
+            between()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        end.record()
+        end.synchronize()
+        ms.append(start.elapsed_time(end))
+    ms = ms[1:]
+    return sum(ms) / len(ms) * 1e3, min(ms) * 1e3   # microseconds
+
+
+def cpu_baseline(cfg, data, bytes_total, budget_s):
+    """The oracle (a scalar C restatement, OpenMP over tokens) timed on this
+    host's cores on the same workload: whole steps until the budget is spent."""
+    import torch
+    from oracle import oracle
+    threads = min(16, os.cpu_count() or 1)
+    oracle.set_threads(threads)
+    R = cfg.num_ranks
+    nt = [cfg.tokens_per_rank] * R
+    eo = torch.empty((R, cfg.num_local_experts, R * cfg.max_tokens, cfg.hidden), dtype=torch.bfloat16)
+    times_d, times_c = [], []
+    t_begin = time.perf_counter()
+    reps = 0
+    while reps < 2 or (time.perf_counter() - t_begin < budget_s and reps < 40):
+        t0 = time.perf_counter()
+        d = oracle.dispatch(data["x"], data["topk_idx"], nt, cfg.max_tokens, cfg.num_experts, cfg.use_fp8, poison=None)
+        t1 = time.perf_counter()
+        oracle.combine(eo, data["topk_idx"], data["topk_weights"], d["src_info"], d["layout_range"], nt,
+                       cfg.max_tokens, cfg.num_experts)
+        t2 = time.perf_counter()
+        if reps > 0:                                   # first repetition pages the buffers in
+            times_d.append(t1 - t0)
+            times_c.append(t2 - t1)
+        reps += 1
+    td, tc = sum(times_d) / len(times_d), sum(times_c) / len(times_c)
+    return {
+        "value": round(bytes_total / (td + tc) / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{len(times_d)} whole steps of the same workload ({cfg.name}, all {R} logical ranks), "
+                  f"first step dropped",
+        "dispatch_us": round(td * 1e6, 1),
+        "combine_us": round(tc * 1e6, 1),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the one-GPU path only: the expert-parallel world is emulated as logical ranks "
+              "inside one MI355X's HBM; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from mooncake_amd import _lib
+    from mooncake_amd.harness import WorldHarness
+    from mooncake_amd.workloads import CONFIGS, algorithmic_bytes, generate
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    cfg = CONFIGS[args.config]
+    data = generate(cfg, seed=args.seed)
+    S = int((data["topk_idx"] >= 0).sum())
+    alg = algorithmic_bytes(cfg, S)
+
+    h = WorldHarness(cfg, device="cuda:0")
+    opts = {}
+    for o in args.opt:
+        k, v = o.split("=")
+        h.world.set_option(k, int(v))
+        opts[k] = int(v)
+    h.load(data)
+    h.alloc_dispatch_outputs()
+    h.alloc_combine_io()
+    h.dispatch()
+    h.fill_expert_out_from_recv()          # expert outputs = dequantised dispatched rows
+    torch.cuda.synchronize()
+
+    def step():
+        h.dispatch()
+        h.combine()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    step_gbps = (alg["dispatch"] + alg["combine"]) / (elapsed / args.steps) / 1e9
+
+    # per-call and per-kernel device times (events on the launch stream); a
+    # 512 MB write before every sample keeps any launch from starting on a
+    # cache warmed by its own previous run
+    flush = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.int32, device="cuda:0")
+    it = args.kernel_iters
+    d_us, _ = time_kernel(h.dispatch, it, flush.zero_)
+    c_us, _ = time_kernel(h.combine, it, flush.zero_)
+    lay_us, _ = time_kernel(lambda: h.dispatch(phases=_lib.PHASE_LAYOUT), it, flush.zero_)
+    pack_us, pack_min = time_kernel(lambda: h.dispatch(phases=_lib.PHASE_DATA), it, flush.zero_)
+    res_us, _ = time_kernel(lambda: h.combine(phases=_lib.PHASE_LAYOUT), it, flush.zero_)
+    red_us, red_min = time_kernel(lambda: h.combine(phases=_lib.PHASE_DATA), it, flush.zero_)
+    del flush
+
+    kernels = {
+        "pack": {"us": round(pack_us, 2), "min_us": round(pack_min, 2), "bytes": alg["dispatch"],
+                 "GBps": round(alg["dispatch"] / pack_us / 1e3, 1)},
+        "reduce": {"us": round(red_us, 2), "min_us": round(red_min, 2), "bytes": alg["combine"],
+                   "GBps": round(alg["combine"] / red_us / 1e3, 1)},
+        "layout": {"us": round(lay_us, 2)},
+        "resolve": {"us": round(res_us, 2)},
+    }
+    # the dominant kernel is the one the step spends most time in
+    dom = "reduce" if red_us >= pack_us else "pack"
+    achieved = kernels[dom]["GBps"]
+    out = {
+        "metric": METRIC,
+        "value": round(step_gbps, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3 dispatch payload (f32 scale math), bf16 combine with f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": cfg.name, "num_ranks": cfg.num_ranks, "tokens_per_rank": cfg.tokens_per_rank,
+                   "hidden": cfg.hidden, "num_experts": cfg.num_experts, "num_topk": cfg.num_topk,
+                   "use_fp8": cfg.use_fp8, "valid_selections": S, "seed": args.seed, "options": opts},
+        "pct_of_hbm_peak": round(step_gbps / HBM_PEAK_GBPS * 100, 2),
+        "dispatch_us": round(d_us, 2),
+        "combine_us": round(c_us, 2),
+        "tokens_per_s": round(cfg.total_tokens / ((d_us + c_us) * 1e-6), 1),
+        "algorithmic_bytes": alg,
+        "kernels": kernels,
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, data, alg["dispatch"] + alg["combine"], args.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

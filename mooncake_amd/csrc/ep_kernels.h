@@ -43,6 +43,23 @@ struct TableChunk {
     uint64_t v[kTableChunk];
 };
 
+// What the routing kernels hand to the data kernels: one fully resolved entry
+// per (rank, token, k) selection.  An entry is valid for the launch whose
+// stamp it carries, so entries that no routing thread visits (masked or
+// out-of-range experts, selections absent from a handle) need no clearing pass.
+struct DispatchRoute {      // 32 bytes
+    uint64_t row;           // byte address of the destination payload row
+    uint64_t scale;         // byte address of scales[le][0][row] (fp8)
+    uint32_t stamp;
+    uint32_t pad[3];
+};
+
+struct CombineRoute {       // 16 bytes
+    uint64_t src;           // byte address of the expert-output row
+    float weight;
+    uint32_t stamp;
+};
+
 struct Dims {
     int R;            // logical ranks
     int E;            // experts
@@ -55,26 +72,40 @@ struct Dims {
 // Tuning knobs, settable at run time for measurement sweeps.
 struct Tuning {
     int layout_block = 1024;   // threads per expert block in the layout kernel
+    int layout_rotate = 1;     // start each expert block at its own offset into the selection list
     int pack_variant = 0;      // 0: 32 B/lane loads, 16 B stores; 1: two coalesced 16 B loads, 8 B stores
     int pack_waves = 4;        // waves per block in the pack kernel
-    int scale_mode = 0;        // 0: scatter scales from the pack kernel; 1: staged + transposing pass
+    int pack_nt = 3;           // bit 0: streaming (nontemporal) loads, bit 1: streaming stores
+    int pack_uniform = 1;      // take x addresses from kernel arguments when the ranks' x are evenly spaced
+    int scale_mode = 1;        // 0: scatter scales from the pack kernel; 1: staged + transposing pass
     int combine_chunks = 1;    // 16-byte chunks per lane in the combine kernel
     int combine_waves = 4;     // waves per block in the combine kernel
-    int nontemporal = 0;       // bit 0: streaming loads, bit 1: streaming stores
+    int combine_nt = 3;        // bit 0: streaming loads, bit 1: streaming stores
+};
+
+// Per-launch inputs of the pack kernel beyond the rank table.
+struct PackLaunch {
+    uint64_t x_base = 0;        // nonzero: rank r's x is x_base + r * x_stride and every rank has uniform_tokens
+    int64_t x_stride = 0;
+    int uniform_tokens = 0;
+    float* scale_stage = nullptr;   // [R * max_tokens, H / 128] staging rows for fp8 scales
 };
 
 hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_words, hipStream_t stream);
 
-hipError_t launch_layout(const uint64_t* d_tbl, int32_t* d_slot_map, const Dims& d, const Tuning& t, hipStream_t stream);
-hipError_t launch_pack(const uint64_t* d_tbl, const int32_t* d_slot_map, float* d_scale_stage, const Dims& d,
-                       bool use_fp8, const Tuning& t, hipStream_t stream);
-hipError_t launch_resolve(const uint64_t* d_tbl, int32_t* d_slot_map, const Dims& d, const Tuning& t,
-                          hipStream_t stream);
-hipError_t launch_reduce(const uint64_t* d_tbl, const int32_t* d_slot_map, const void* d_zero_row, const Dims& d,
+hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, uint32_t stamp, const Dims& d, bool use_fp8,
                          const Tuning& t, hipStream_t stream);
+hipError_t launch_pack(const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp, const PackLaunch& pl,
+                       const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream);
+hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, const Dims& d,
+                          const Tuning& t, hipStream_t stream);
+hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const void* d_zero_row,
+                         const Dims& d, const Tuning& t, hipStream_t stream);
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 hipError_t launch_fill_u32(void* dst, uint32_t value, size_t words, hipStream_t stream);
 
-size_t layout_lds_bytes(const Dims& d, bool* masks_in_lds);
+// selections (R * max_tokens * K) the layout kernel can hold ballots for in LDS
+constexpr size_t kMaxLayoutLdsBytes = 144 * 1024;
+size_t layout_lds_bytes(const Dims& d);
 
 }  // namespace mcep

@@ -5,7 +5,7 @@
 //
 //   layout_kernel   routing layout: per-expert histogram, per-(expert, source
 //                   rank) ranges by prefix sum, source-index map and the
-//                   (rank, token, k) -> packed-row map.  Restates the count
+//                   resolved destination of every (rank, token, k) selection.  Restates the count
 //                   path and the slot assignment of the reference's dispatch
 //                   (mooncake-ep/src/mooncake_ep_kernel.cu:274, :319-356,
 //                   :417-437) in a deterministic order: source rank ascending,
@@ -16,8 +16,9 @@
 //                   (mooncake_ep_kernel.cu:183-186, :233-264), K row stores
 //                   straight into [local expert, R*max, hidden]
 //                   (the reference needs two hops, :273-306 then :442-466).
-//   resolve_kernel  combine's handle (src_info, layout_range) -> packed row of
-//                   each (token, k) (data flow of mooncake_ep_kernel.cu:611-637).
+//   resolve_kernel  combine's handle (src_info, layout_range) -> source row and
+//                   weight of each (token, k) (data flow of
+//                   mooncake_ep_kernel.cu:611-637).
 //   reduce_kernel   per token: fp32 fused multiply-add over its top-k expert
 //                   rows in k order, round to nearest even bf16
 //                   (mooncake_ep_kernel.cu:711-753).
@@ -98,114 +99,133 @@ __global__ void table_write_kernel(uint64_t* dst, TableChunk chunk, int n) {
 // ---------------------------------------------------------------------------
 // routing layout
 // ---------------------------------------------------------------------------
-// One block per global expert e.  Selections of a source rank are scanned in
-// flat (token, k) order, 64 per wave step, so a wave's ballot of "selects e"
-// lists that rank's tokens in ascending order (a token names an expert at most
-// once; a repeated expert is counted at its first k only).  Pass 1 keeps the
-// ballots in LDS and counts per source rank; wave 0 turns the counts into
-// begins by prefix sum; pass 2 turns ballot bits into packed rows.
-__device__ __forceinline__ unsigned long long select_mask(const int64_t* idx, int n, int K, int e, int word,
-                                                          int lane) {
-    const int i = word * 64 + lane;
-    const int64_t v = (i < n) ? idx[i] : -1;
-    bool hit = (v == (int64_t)e);
-    if (hit) {
-        const int t = i / K, k = i - t * K;
-        for (int k2 = 0; k2 < k; ++k2)
-            if (idx[t * K + k2] == (int64_t)e) hit = false;
-    }
-    return __ballot(hit);
-}
-
+// One block per global expert e.  The world's selections form a flat list of
+// 64-entry words, rank-major with a fixed number of words per rank, so that a
+// wave's ballot of "selects e" over one word lists tokens of one source rank in
+// ascending order.  (A token is expected to name an expert at most once; if it
+// names one twice, each occurrence gets its own row, as in the reference
+// kernel, which sends once per k: mooncake_ep_kernel.cu:230,273.)
+//   pass 1  ballots of every word -> LDS.  Each block starts at its own offset
+//           into the list: all E blocks read the same R*T*K indices, and
+//           without the rotation they would all ask the same L2 channel for
+//           the same line at the same time.
+//   scan    exclusive prefix of the per-word popcounts = packed row of the
+//           first hit of each word; rank boundaries give (begin, count).
+//   pass 2  ballot bits -> src_info entries and resolved destination routes.
+template <bool FP8>
 __global__ __launch_bounds__(1024) void layout_kernel(const uint64_t* __restrict__ tbl,
-                                                       int32_t* __restrict__ slot_map, int R, int E, int K,
-                                                       int max_tokens, int words_per_rank, int masks_in_lds) {
+                                                       DispatchRoute* __restrict__ routes, uint32_t stamp, int R,
+                                                       int E, int K, int H, int max_tokens, int words_per_rank,
+                                                       int rotate) {
     extern __shared__ unsigned long long lds[];
-    unsigned long long* masks = lds;
-    int* cnt = (int*)(lds + (masks_in_lds ? (size_t)R * words_per_rank : 0));
-    int* beg = cnt + R;
+    const int W = R * words_per_rank;
+    unsigned long long* masks = lds;                       // [W]
+    int* wbeg = (int*)(lds + W);                           // [W + 1]
+    int* wave_tot = wbeg + W + 1;                          // [16]
 
     const int e = blockIdx.x;
     const int L = E / R, q = e / L, le = e - q * L;
-    const int lane = wave_lane(), wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    // the wave index is wave-uniform: keep it (and all word / rank arithmetic
+    // that follows from it) in scalar registers
+    const int lane = wave_lane(), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
     const int64_t RM = (int64_t)R * max_tokens;
 
-    // a rank that takes no part in this dispatch receives nothing
-    if (tbl[DF_RECV_X * R + q] == 0) return;
+    // a rank that takes no part in this dispatch receives nothing; routes
+    // towards it keep an old stamp and are skipped by the pack kernel
+    const uint64_t recv_x = tbl[DF_RECV_X * R + q];
+    if (recv_x == 0) return;
     int32_t* recv_count = (int32_t*)tbl[DF_RECV_COUNT * R + q];
     int32_t* src_info = (int32_t*)tbl[DF_SRC_INFO * R + q] + (int64_t)le * RM;
     int64_t* layout_range = (int64_t*)tbl[DF_LAYOUT_RANGE * R + q] + (int64_t)le * R;
 
-    for (int r = wave; r < R; r += nwaves) {
+    // An item is a run of up to U consecutive words of one rank: one rank-table
+    // lookup and one division per item, U independent loads in flight per lane.
+    constexpr int U = 8;
+    const int items_per_rank = (words_per_rank + U - 1) / U;
+    const int items = R * items_per_rank;
+    const int start = rotate ? (int)(((long long)e * items) / E) : 0;
+    for (int it = wave; it < items; it += nwaves) {
+        int item = it + start;
+        if (item >= items) item -= items;
+        const int r = item / items_per_rank, w0 = (item - r * items_per_rank) * U;
         const int n = (int)tbl[DF_NUM_TOKENS * R + r] * K;
         const int64_t* idx = (const int64_t*)tbl[DF_TOPK_IDX * R + r];
-        int c = 0;
-        const int nwords = (n + 63) >> 6;
-        int w = 0;
-        for (; w + 4 <= nwords; w += 4) {
-            // four independent loads in flight per lane
-            unsigned long long m0 = select_mask(idx, n, K, e, w + 0, lane);
-            unsigned long long m1 = select_mask(idx, n, K, e, w + 1, lane);
-            unsigned long long m2 = select_mask(idx, n, K, e, w + 2, lane);
-            unsigned long long m3 = select_mask(idx, n, K, e, w + 3, lane);
-            if (masks_in_lds && lane == 0) {
-                unsigned long long* mw = masks + (size_t)r * words_per_rank + w;
-                mw[0] = m0; mw[1] = m1; mw[2] = m2; mw[3] = m3;
-            }
-            c += __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3);
-        }
-        for (; w < nwords; ++w) {
-            unsigned long long m = select_mask(idx, n, K, e, w, lane);
-            if (masks_in_lds && lane == 0) masks[(size_t)r * words_per_rank + w] = m;
-            c += __popcll(m);
-        }
-        if (lane == 0) cnt[r] = c;
-    }
-    __syncthreads();
-
-    if (wave == 0) {
-        int running = 0;
-        for (int r0 = 0; r0 < R; r0 += 64) {
-            const int r = r0 + lane;
-            const int v = (r < R) ? cnt[r] : 0;
-            int incl = v;
+        int64_t v[U];
 #pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int u = __shfl_up(incl, d);
-                if (lane >= d) incl += u;
-            }
-            const int b = running + incl - v;
-            if (r < R) {
-                beg[r] = b;
-                // count in the low half, begin in the high half; an empty pair is 0
-                layout_range[r] = v ? (((int64_t)b << 32) | (int64_t)v) : 0;
-            }
-            running += __shfl(incl, 63);
+        for (int u = 0; u < U; ++u) {
+            const int i = (w0 + u) * 64 + lane;
+            v[u] = (w0 + u < words_per_rank && i < n) ? idx[i] : -1;
         }
-        if (lane == 0) recv_count[le] = running;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (w0 + u >= words_per_rank) break;
+            const unsigned long long m = __ballot(v[u] == (int64_t)e);
+            if (lane == 0) masks[r * words_per_rank + w0 + u] = m;
+        }
     }
     __syncthreads();
 
-    for (int r = wave; r < R; r += nwaves) {
-        const int n = (int)tbl[DF_NUM_TOKENS * R + r] * K;
-        const int64_t* idx = (const int64_t*)tbl[DF_TOPK_IDX * R + r];
-        int32_t* smap = slot_map + (int64_t)r * max_tokens * K;
-        int run = beg[r];
-        const int nwords = (n + 63) >> 6;
-        for (int w = 0; w < nwords; ++w) {
-            const unsigned long long m =
-                masks_in_lds ? masks[(size_t)r * words_per_rank + w] : select_mask(idx, n, K, e, w, lane);
+    // block-wide exclusive scan of the per-word hit counts
+    int carry = 0;
+    for (int base = 0; base < W; base += blockDim.x) {
+        const int gi = base + threadIdx.x;
+        const int c = (gi < W) ? __popcll(masks[gi]) : 0;
+        int incl = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+        if (lane == 63) wave_tot[wave] = incl;
+        __syncthreads();
+        int before = carry;
+        for (int w2 = 0; w2 < wave; ++w2) before += wave_tot[w2];
+        if (gi < W) wbeg[gi] = before + incl - c;
+        int total = 0;
+        for (int w2 = 0; w2 < nwaves; ++w2) total += wave_tot[w2];
+        carry += total;
+        __syncthreads();
+    }
+    // A block holds RM rows.  Distinct experts per token can never exceed that;
+    // rows past it (possible only with repeated experts) are dropped.
+    const int cap = (int)(RM < 0x7fffffff ? RM : 0x7fffffff);
+    if (threadIdx.x == 0) {
+        wbeg[W] = carry;
+        recv_count[le] = carry < cap ? carry : cap;
+    }
+    __syncthreads();
+    for (int r = threadIdx.x; r < R; r += blockDim.x) {
+        int b = wbeg[r * words_per_rank], b2 = wbeg[(r + 1) * words_per_rank];
+        b = b < cap ? b : cap;
+        b2 = b2 < cap ? b2 : cap;
+        const int c = b2 - b;
+        // count in the low half, begin in the high half; an empty pair is 0
+        layout_range[r] = c ? (((int64_t)b << 32) | (int64_t)c) : 0;
+    }
+
+    const uint64_t row_bytes = (uint64_t)H * (FP8 ? 1 : 2);
+    const uint64_t row0 = recv_x + (uint64_t)le * RM * row_bytes;
+    const uint64_t scale0 = FP8 ? tbl[DF_RECV_SCALES * R + q] + (uint64_t)le * (H / 128) * RM * 4 : 0;
+    for (int it = wave; it < items; it += nwaves) {
+        const int r = it / items_per_rank, w0 = (it - r * items_per_rank) * U;
+        for (int u = 0; u < U && w0 + u < words_per_rank; ++u) {
+            const int gi = r * words_per_rank + w0 + u;
+            const unsigned long long m = masks[gi];
             if (m == 0) continue;
             if ((m >> lane) & 1ull) {
-                const int pos = run + __popcll(m & ((1ull << lane) - 1ull));
-                const int i = w * 64 + lane;
-                const int t = i / K, k = i - t * K;
-                src_info[pos] = t;
-                smap[i] = pos;
-                for (int k2 = k + 1; k2 < K; ++k2)
-                    if (idx[t * K + k2] == (int64_t)e) smap[t * K + k2] = pos;
+                const int pos = wbeg[gi] + __popcll(m & ((1ull << lane) - 1ull));
+                if (pos < cap) {
+                    const int i = (w0 + u) * 64 + lane;
+                    const int t = i / K, k = i - t * K;
+                    src_info[pos] = t;
+                    DispatchRoute rt;
+                    rt.row = row0 + (uint64_t)pos * row_bytes;
+                    rt.scale = FP8 ? scale0 + (uint64_t)pos * 4 : 0;
+                    rt.stamp = stamp;
+                    rt.pad[0] = rt.pad[1] = rt.pad[2] = 0;
+                    routes[((int64_t)r * max_tokens + t) * K + k] = rt;
+                }
             }
-            run += __popcll(m);
         }
     }
 }
@@ -213,32 +233,58 @@ __global__ __launch_bounds__(1024) void layout_kernel(const uint64_t* __restrict
 // ---------------------------------------------------------------------------
 // dispatch pack
 // ---------------------------------------------------------------------------
-// One wave per (token, 1024-element slab).  Lanes 0..K-1 resolve the K
-// destination rows; the row slab is read once, quantised in registers and
-// stored K times.
+// One wave per (token, 1024-element slab).  Lanes 0..K-1 fetch the K resolved
+// destinations; the row slab is read once, quantised in registers and stored
+// K times.
 struct PackDest {
     uint64_t row;     // byte address of the destination row, 0 = no store
     uint64_t scale;   // byte address of scales[le][0][slot] (fp8)
 };
 
-template <bool FP8>
-__device__ __forceinline__ PackDest pack_resolve(const uint64_t* __restrict__ tbl,
-                                                 const int32_t* __restrict__ slot_map, int R, int E, int K,
-                                                 int max_tokens, int H, int r, int t, int lane) {
-    PackDest d = {0, 0};
-    if (lane < K) {
-        const int64_t e64 = ((const int64_t*)tbl[DF_TOPK_IDX * R + r])[t * K + lane];
-        if (e64 >= 0 && e64 < (int64_t)E) {
-            const int e = (int)e64, L = E / R, q = e / L, le = e - q * L;
-            const int slot = slot_map[((int64_t)r * max_tokens + t) * K + lane];
-            const int64_t RM = (int64_t)R * max_tokens;
-            const uint64_t base = tbl[DF_RECV_X * R + q];
-            if (base != 0) {
-                d.row = base + (uint64_t)(((int64_t)le * RM + slot) * H) * (FP8 ? 1 : 2);
-                if (FP8) d.scale = tbl[DF_RECV_SCALES * R + q] + (uint64_t)((int64_t)le * (H / 128) * RM + slot) * 4;
-            }
-        }
+// Where a wave finds its token row.  When every rank's x is the same distance
+// from the previous rank's and all ranks hold the same number of tokens, the
+// address comes from kernel arguments alone; otherwise from the rank table
+// (one more dependent scalar load before the row loads can be issued).
+struct PackSource {
+    uint64_t x_base;      // rank 0's x when uniform, else 0
+    int64_t x_stride;     // bytes between consecutive ranks' x
+    int tokens;           // every rank's token count when uniform
+};
+
+__device__ __forceinline__ const char* pack_source_row(const uint64_t* __restrict__ tbl, const PackSource& src, int R,
+                                                       int H, int r, int t, bool* in_range) {
+    if (src.x_base != 0) {
+        *in_range = t < src.tokens;
+        return (const char*)(src.x_base + (uint64_t)((int64_t)r * src.x_stride)) + (int64_t)t * H * 2;
     }
+    *in_range = t < (int)tbl[DF_NUM_TOKENS * R + r];
+    return (const char*)tbl[DF_X * R + r] + (int64_t)t * H * 2;
+}
+
+struct PackRouteRaw {
+    uint4 a, b;
+};
+
+// issue the route loads (no dependency on anything but the task index) ...
+__device__ __forceinline__ PackRouteRaw pack_route_issue(const DispatchRoute* __restrict__ routes, int K,
+                                                         int max_tokens, int r, int t, int lane) {
+    PackRouteRaw raw = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    if (lane < K) {
+        const uint4* p = (const uint4*)(routes + ((int64_t)r * max_tokens + t) * K + lane);
+        raw.a = p[0];
+        raw.b = p[1];
+    }
+    return raw;
+}
+
+// ... and consume them after the row loads are in flight.  The empty asm keeps
+// the compiler from fetching the stamp first and the rest behind a branch.
+__device__ __forceinline__ PackDest pack_route_finish(PackRouteRaw raw, uint32_t stamp, int K, int lane) {
+    asm volatile("" : "+v"(raw.a.x), "+v"(raw.a.y), "+v"(raw.a.z), "+v"(raw.a.w), "+v"(raw.b.x));
+    const bool ok = (lane < K) && (raw.b.x == stamp);
+    PackDest d;
+    d.row = ok ? (((uint64_t)raw.a.y << 32) | raw.a.x) : 0;
+    d.scale = ok ? (((uint64_t)raw.a.w << 32) | raw.a.z) : 0;
     return d;
 }
 
@@ -246,25 +292,29 @@ __device__ __forceinline__ PackDest pack_resolve(const uint64_t* __restrict__ tb
 // a 128-element scale group is 8 lanes.
 template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restrict__ tbl,
-                                                        const int32_t* __restrict__ slot_map, int R, int E, int K,
-                                                        int max_tokens, int H, int slabs, int Tgrid,
+                                                        const DispatchRoute* __restrict__ routes, uint32_t stamp,
+                                                        PackSource src, float* __restrict__ scale_stage, int R,
+                                                        int K, int max_tokens, int H, int slabs, int Tgrid,
                                                         int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
-    if (t >= (int)tbl[DF_NUM_TOKENS * R + r]) return;
+    const PackRouteRaw raw = pack_route_issue(routes, K, max_tokens, r, t, lane);
+    bool in_range;
+    const char* xtok = pack_source_row(tbl, src, R, H, r, t, &in_range);
+    if (!in_range) return;
 
     const int elem0 = s * 1024 + lane * 16;
     const bool active = elem0 < H;
-    const char* xrow = (const char*)tbl[DF_X * R + r] + ((int64_t)t * H + (active ? elem0 : 0)) * 2;
+    const char* xrow = xtok + (int64_t)(active ? elem0 : 0) * 2;
     uint4 a = make_uint4(0, 0, 0, 0), b = a;
     if (active) {
         a = load16<NTL>(xrow);
         b = load16<NTL>(xrow + 16);
     }
-    const PackDest dst = pack_resolve<true>(tbl, slot_map, R, E, K, max_tokens, H, r, t, lane);
+    const PackDest dst = pack_route_finish(raw, stamp, K, lane);
 
     float f[16];
     const uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
@@ -291,13 +341,18 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
     const uint4 out = make_uint4(o[0], o[1], o[2], o[3]);
     const int64_t scale_off = (int64_t)(elem0 >> 7) * ((int64_t)R * max_tokens) * 4;
     const bool scale_lane = active && ((lane & 7) == 0);
+    // staged: the token's scales go to one contiguous row, a second kernel
+    // moves them into the column-major output with coalesced stores
+    if (scale_stage != nullptr && scale_lane)
+        scale_stage[((int64_t)r * max_tokens + t) * (H >> 7) + (elem0 >> 7)] = scale_inv;
+    const bool scatter_scales = scale_lane && scale_stage == nullptr;
 
     for (int k = 0; k < K; ++k) {
         const uint64_t row = read_lane_u64(dst.row, k);
         const uint64_t sc = read_lane_u64(dst.scale, k);
         if (row == 0) continue;
         if (active) store16<NTS>((void*)(row + elem0), out);
-        if (scale_lane) *(float*)(sc + scale_off) = scale_inv;
+        if (scatter_scales) *(float*)(sc + scale_off) = scale_inv;
     }
 }
 
@@ -306,17 +361,21 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
 // stores are 8 bytes per lane.
 template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __restrict__ tbl,
-                                                              const int32_t* __restrict__ slot_map, int R, int E,
-                                                              int K, int max_tokens, int H, int slabs, int Tgrid,
+                                                              const DispatchRoute* __restrict__ routes,
+                                                              uint32_t stamp, PackSource src,
+                                                              float* __restrict__ scale_stage, int R, int K,
+                                                              int max_tokens, int H, int slabs, int Tgrid,
                                                               int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
-    if (t >= (int)tbl[DF_NUM_TOKENS * R + r]) return;
+    const PackRouteRaw raw = pack_route_issue(routes, K, max_tokens, r, t, lane);
+    bool in_range;
+    const char* xbase = pack_source_row(tbl, src, R, H, r, t, &in_range);
+    if (!in_range) return;
 
-    const char* xbase = (const char*)tbl[DF_X * R + r] + (int64_t)t * H * 2;
     int elem[2];
     bool active[2];
     uint4 v[2];
@@ -327,7 +386,7 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
         v[p] = make_uint4(0, 0, 0, 0);
         if (active[p]) v[p] = load16<NTL>(xbase + (int64_t)elem[p] * 2);
     }
-    const PackDest dst = pack_resolve<true>(tbl, slot_map, R, E, K, max_tokens, H, r, t, lane);
+    const PackDest dst = pack_route_finish(raw, stamp, K, lane);
 
     uint2 out[2];
     float scale_inv[2];
@@ -353,6 +412,13 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
         out[p] = make_uint2((uint32_t)w0, (uint32_t)w1);
     }
     const int64_t RM4 = (int64_t)R * max_tokens * 4;
+    const bool scale_lane = (lane & 15) == 0;
+    if (scale_stage != nullptr && scale_lane) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+            if (active[p]) scale_stage[((int64_t)r * max_tokens + t) * (H >> 7) + (elem[p] >> 7)] = scale_inv[p];
+    }
+    const bool scatter_scales = scale_lane && scale_stage == nullptr;
 
     for (int k = 0; k < K; ++k) {
         const uint64_t row = read_lane_u64(dst.row, k);
@@ -362,7 +428,7 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
         for (int p = 0; p < 2; ++p) {
             if (active[p]) {
                 store8<NTS>((void*)(row + elem[p]), out[p]);
-                if ((lane & 15) == 0) *(float*)(sc + (int64_t)(elem[p] >> 7) * RM4) = scale_inv[p];
+                if (scatter_scales) *(float*)(sc + (int64_t)(elem[p] >> 7) * RM4) = scale_inv[p];
             }
         }
     }
@@ -371,17 +437,20 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
 // bf16: plain row copy, two unit-stride 16-byte pieces per lane.
 template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restrict__ tbl,
-                                                         const int32_t* __restrict__ slot_map, int R, int E, int K,
-                                                         int max_tokens, int H, int slabs, int Tgrid,
+                                                         const DispatchRoute* __restrict__ routes, uint32_t stamp,
+                                                         PackSource src, float* __restrict__ /*scale_stage*/, int R,
+                                                         int K, int max_tokens, int H, int slabs, int Tgrid,
                                                          int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
-    if (t >= (int)tbl[DF_NUM_TOKENS * R + r]) return;
+    const PackRouteRaw raw = pack_route_issue(routes, K, max_tokens, r, t, lane);
+    bool in_range;
+    const char* xbase = pack_source_row(tbl, src, R, H, r, t, &in_range);
+    if (!in_range) return;
 
-    const char* xbase = (const char*)tbl[DF_X * R + r] + (int64_t)t * H * 2;
     int64_t off[2];
     bool active[2];
     uint4 v[2];
@@ -393,7 +462,7 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
         v[p] = make_uint4(0, 0, 0, 0);
         if (active[p]) v[p] = load16<NTL>(xbase + off[p]);
     }
-    const PackDest dst = pack_resolve<false>(tbl, slot_map, R, E, K, max_tokens, H, r, t, lane);
+    const PackDest dst = pack_route_finish(raw, stamp, K, lane);
 
     for (int k = 0; k < K; ++k) {
         const uint64_t row = read_lane_u64(dst.row, k);
@@ -404,83 +473,163 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
     }
 }
 
-// ---------------------------------------------------------------------------
-// combine
-// ---------------------------------------------------------------------------
-// One wave per token: for each k, the (expert, source rank) block named by
-// layout_range is searched for the token index, 64 src_info entries per step.
-__global__ __launch_bounds__(256) void resolve_kernel(const uint64_t* __restrict__ tbl,
-                                                       int32_t* __restrict__ slot_map, int R, int E, int K,
-                                                       int max_tokens, int Tgrid, int total_tasks) {
+// Staged scales -> column-major output.  kTransposeWaves waves per expert,
+// each taking 64 packed rows at a time: a lane finds its row's source token
+// (src_info, and the source rank from the expert's ranges, fetched once per
+// wave), reads that token's H/128 scales as contiguous 16-byte pieces - a
+// batch of them in flight at once - and stores them so that the wave writes
+// 64 consecutive floats per scale group.
+constexpr int kTransposeWaves = 8;
+
+__global__ __launch_bounds__(256) void scale_transpose_kernel(const uint64_t* __restrict__ tbl,
+                                                               const float* __restrict__ scale_stage, int R, int E,
+                                                               int G, int max_tokens, int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
-    const int r = task / Tgrid, t = task - r * Tgrid;
-    if (t >= (int)tbl[CF_NUM_TOKENS * R + r]) return;
-    const int L = E / R;
+    const int e = task / kTransposeWaves, wi = task - e * kTransposeWaves;
+    const int L = E / R, q = e / L, le = e - q * L;
+    if (tbl[DF_RECV_X * R + q] == 0) return;
+    const int count = ((const int32_t*)tbl[DF_RECV_COUNT * R + q])[le];
+    if (wi * 64 >= count) return;
     const int64_t RM = (int64_t)R * max_tokens;
-    const int64_t* idx = (const int64_t*)tbl[CF_TOPK_IDX * R + r] + (int64_t)t * K;
-    int32_t* smap = slot_map + ((int64_t)r * max_tokens + t) * K;
+    const int32_t* src_info = (const int32_t*)tbl[DF_SRC_INFO * R + q] + (int64_t)le * RM;
+    const int64_t* ranges = (const int64_t*)tbl[DF_LAYOUT_RANGE * R + q] + (int64_t)le * R;
+    float* out = (float*)tbl[DF_RECV_SCALES * R + q] + (int64_t)le * G * RM;
 
-    for (int k = 0; k < K; ++k) {
-        const int64_t e64 = idx[k];
-        int found = -1;
-        if (e64 >= 0 && e64 < (int64_t)E) {
-            const int e = (int)e64, q = e / L, le = e - q * L;
-            const int64_t* lrp = (const int64_t*)tbl[CF_LAYOUT_RANGE * R + q];
-            const int32_t* sip = (const int32_t*)tbl[CF_SRC_INFO * R + q];
-            if (lrp != nullptr && sip != nullptr) {
-                const int64_t lr = lrp[(int64_t)le * R + r];
-                int count = (int)(lr & 0xffffffffll);
-                int begin = (int)(lr >> 32);
-                if (begin < 0 || count < 0 || (int64_t)begin + count > RM) count = 0;   // malformed handle
-                sip += (int64_t)le * RM + begin;
-                for (int i0 = 0; i0 < count; i0 += 64) {
-                    const int i = i0 + lane;
-                    const bool hit = (i < count) && (sip[i] == t);
-                    const unsigned long long m = __ballot(hit);
-                    if (m) {
-                        found = begin + i0 + (__ffsll((long long)m) - 1);
-                        break;
+    for (int row0 = wi * 64; row0 < count; row0 += kTransposeWaves * 64) {
+        const int row = row0 + lane;
+        const bool valid = row < count;
+        const int t = valid ? src_info[row] : 0;
+        // source rank of the row: the range that contains it (ranges held one per lane)
+        int r = 0;
+        for (int rb = 0; rb < R; rb += 64) {
+            const int64_t mine = (rb + lane < R) ? ranges[rb + lane] : 0;
+            const int nr = (R - rb < 64) ? (R - rb) : 64;
+            for (int j = 0; j < nr; ++j) {
+                const int c = __builtin_amdgcn_readlane((int)(uint32_t)mine, j);
+                const int b = __builtin_amdgcn_readlane((int)(uint32_t)(mine >> 32), j);
+                if (c != 0 && row >= b && row < b + c) r = rb + j;
+            }
+        }
+        const float* sp = scale_stage + ((int64_t)r * max_tokens + t) * G;
+        float* dp = out + row;
+        int g = 0;
+        if ((G & 3) == 0) {
+            constexpr int B = 8;   // 16-byte loads in flight per lane
+            for (; g + 4 * B <= G; g += 4 * B) {
+                float4 v[B];
+#pragma unroll
+                for (int j = 0; j < B; ++j) v[j] = valid ? *(const float4*)(sp + g + 4 * j) : make_float4(0, 0, 0, 0);
+                if (valid) {
+#pragma unroll
+                    for (int j = 0; j < B; ++j) {
+                        dp[(int64_t)(g + 4 * j + 0) * RM] = v[j].x;
+                        dp[(int64_t)(g + 4 * j + 1) * RM] = v[j].y;
+                        dp[(int64_t)(g + 4 * j + 2) * RM] = v[j].z;
+                        dp[(int64_t)(g + 4 * j + 3) * RM] = v[j].w;
                     }
                 }
             }
+            for (; g < G; g += 4) {
+                if (valid) {
+                    const float4 v = *(const float4*)(sp + g);
+                    dp[(int64_t)(g + 0) * RM] = v.x;
+                    dp[(int64_t)(g + 1) * RM] = v.y;
+                    dp[(int64_t)(g + 2) * RM] = v.z;
+                    dp[(int64_t)(g + 3) * RM] = v.w;
+                }
+            }
         }
-        if (lane == 0) smap[k] = found;
+        if (valid)
+            for (; g < G; ++g) dp[(int64_t)g * RM] = sp[g];
     }
 }
 
-// One wave per (token, slab of CH * 512 elements).  Lanes 0..KMAX-1 resolve
-// the K source rows (a masked, inactive or unknown selection reads a zero row
-// with weight 0, which leaves the fp32 accumulator unchanged), then every
-// lane issues all KMAX * CH 16-byte loads before the first multiply-add.
+// ---------------------------------------------------------------------------
+// combine
+// ---------------------------------------------------------------------------
+// Handle -> routes.  One wave per (expert, token-owner rank) pair: the packed
+// rows [begin, begin + count) of that pair carry the owner's token indices in
+// src_info; each row finds its k in the token's top-k list and leaves the
+// row's address and weight there.  Experts on ranks the owner sees as
+// inactive, and rows of ranks that take no part, leave no route.
+__global__ __launch_bounds__(256) void resolve_kernel(const uint64_t* __restrict__ tbl,
+                                                       CombineRoute* __restrict__ routes, uint32_t stamp, int R,
+                                                       int E, int K, int H, int max_tokens, int total_tasks) {
+    const int lane = wave_lane();
+    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    if (task >= total_tasks) return;
+    const int e = task / R, r = task - e * R;
+    const int L = E / R, q = e / L, le = e - q * L;
+    const int T = (int)tbl[CF_NUM_TOKENS * R + r];
+    if (T == 0) return;
+    const uint64_t base = tbl[CF_X * R + q];
+    const int64_t* lrp = (const int64_t*)tbl[CF_LAYOUT_RANGE * R + q];
+    const int32_t* sip = (const int32_t*)tbl[CF_SRC_INFO * R + q];
+    if (base == 0 || lrp == nullptr || sip == nullptr) return;
+    if (((const int32_t*)tbl[CF_ACTIVE * R + r])[q] == 0) return;   // skip experts on inactive ranks
+    const int64_t RM = (int64_t)R * max_tokens;
+    const int64_t lr = lrp[(int64_t)le * R + r];
+    const int count = (int)(lr & 0xffffffffll), begin = (int)(lr >> 32);
+    if (begin < 0 || count <= 0 || (int64_t)begin + count > RM) return;   // empty or malformed
+    sip += (int64_t)le * RM + begin;
+    const int64_t* idx = (const int64_t*)tbl[CF_TOPK_IDX * R + r];
+    const float* wts = (const float*)tbl[CF_TOPK_W * R + r];
+    CombineRoute* rts = routes + (int64_t)r * max_tokens * K;
+    const uint64_t row0 = base + (uint64_t)((int64_t)le * RM + begin) * H * 2;
+    for (int i = lane; i < count; i += 64) {
+        const int t = sip[i];
+        if (t < 0 || t >= T) continue;
+        for (int k0 = 0; k0 < K; k0 += 4) {
+            int64_t cand[4];
+            float wt[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool in = k0 + j < K;
+                cand[j] = in ? idx[(int64_t)t * K + k0 + j] : -1;
+                wt[j] = in ? wts[(int64_t)t * K + k0 + j] : 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (cand[j] == (int64_t)e) {
+                    CombineRoute rt;
+                    rt.src = row0 + (uint64_t)i * H * 2;
+                    rt.weight = wt[j];
+                    rt.stamp = stamp;
+                    rts[(int64_t)t * K + k0 + j] = rt;
+                }
+            }
+        }
+    }
+}
+
+// One wave per (token, slab of CH * 512 elements).  Lanes 0..K-1 fetch the K
+// routes (a masked, inactive or unknown selection reads a zero row with
+// weight 0, which leaves the fp32 accumulator unchanged), then every lane
+// issues all KMAX * CH 16-byte loads before the first multiply-add.
 template <int KMAX, int CH, bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict__ tbl,
-                                                      const int32_t* __restrict__ slot_map,
-                                                      const void* __restrict__ zero_row, int R, int E, int K,
+                                                      const CombineRoute* __restrict__ routes, uint32_t stamp,
+                                                      const void* __restrict__ zero_row, int R, int K,
                                                       int max_tokens, int H, int slabs, int Tgrid, int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
-    if (t >= (int)tbl[CF_NUM_TOKENS * R + r]) return;
+    // A token slot beyond the rank's count has only stale routes (zero rows);
+    // it is computed like any other and dropped at the store, so that no wave
+    // waits for the rank's token count before it can issue its loads.
+    const int T = (int)tbl[CF_NUM_TOKENS * R + r];
+    char* orow = (char*)tbl[CF_OUT * R + r] + (int64_t)t * H * 2;
 
-    uint64_t src = (uint64_t)zero_row;
-    float w = 0.0f;
-    if (lane < K) {
-        const int64_t e64 = ((const int64_t*)tbl[CF_TOPK_IDX * R + r])[(int64_t)t * K + lane];
-        if (e64 >= 0 && e64 < (int64_t)E) {
-            const int e = (int)e64, L = E / R, q = e / L, le = e - q * L;
-            const int slot = slot_map[((int64_t)r * max_tokens + t) * K + lane];
-            const int live = ((const int32_t*)tbl[CF_ACTIVE * R + r])[q];   // skip experts on inactive ranks
-            const uint64_t base = tbl[CF_X * R + q];
-            if (slot >= 0 && live != 0 && base != 0) {
-                src = base + (uint64_t)(((int64_t)le * R * max_tokens + slot) * H) * 2;
-                w = ((const float*)tbl[CF_TOPK_W * R + r])[(int64_t)t * K + lane];
-            }
-        }
-    }
+    uint4 rt = make_uint4(0, 0, 0, 0);
+    if (lane < K) rt = *(const uint4*)(routes + ((int64_t)r * max_tokens + t) * K + lane);
+    asm volatile("" : "+v"(rt.x), "+v"(rt.y), "+v"(rt.z), "+v"(rt.w));   // one 16-byte load, no branch on the stamp
+    const bool ok = (lane < K) && (rt.w == stamp);
+    const uint64_t src = ok ? (((uint64_t)rt.y << 32) | rt.x) : (uint64_t)zero_row;
+    const float w = ok ? __uint_as_float(rt.z) : 0.0f;
 
     int64_t off[CH];
     bool active[CH];
@@ -501,7 +650,7 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
         for (int c = 0; c < CH; ++c) v[k][c] = load16<NTL>((const void*)(p + off[c]));
     }
 
-    char* orow = (char*)tbl[CF_OUT * R + r] + (int64_t)t * H * 2;
+    if (t >= T) return;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         float acc[8];
@@ -560,83 +709,99 @@ hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_word
     return hipSuccess;
 }
 
-size_t layout_lds_bytes(const Dims& d, bool* masks_in_lds) {
+size_t layout_lds_bytes(const Dims& d) {
     const size_t words_per_rank = ((size_t)d.max_tokens * d.K + 63) / 64;
-    const size_t fixed = (size_t)d.R * 2 * sizeof(int);
-    const size_t with_masks = (size_t)d.R * words_per_rank * 8 + fixed;
-    const bool fits = with_masks <= 60 * 1024;
-    if (masks_in_lds) *masks_in_lds = fits;
-    return fits ? with_masks : fixed;
+    const size_t W = (size_t)d.R * words_per_rank;
+    return W * 8 + (W + 1) * 4 + 16 * 4 + 16;
 }
 
-hipError_t launch_layout(const uint64_t* d_tbl, int32_t* d_slot_map, const Dims& d, const Tuning& t,
-                         hipStream_t stream) {
-    bool in_lds = false;
-    const size_t lds = layout_lds_bytes(d, &in_lds);
+hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, uint32_t stamp, const Dims& d, bool use_fp8,
+                         const Tuning& t, hipStream_t stream) {
+    const size_t lds = layout_lds_bytes(d);
+    if (lds > kMaxLayoutLdsBytes) return hipErrorInvalidValue;
     const int words_per_rank = (int)(((size_t)d.max_tokens * d.K + 63) / 64);
     int block = t.layout_block;
     if (block < 64) block = 64;
     if (block > 1024) block = 1024;
     block &= ~63;
-    hipLaunchKernelGGL(layout_kernel, dim3(d.E), dim3(block), lds, stream, d_tbl, d_slot_map, d.R, d.E, d.K,
-                       d.max_tokens, words_per_rank, in_lds ? 1 : 0);
-    return hipGetLastError();
-}
-
-template <typename Kern>
-static hipError_t launch_wave_tasks(Kern kern, int waves_per_block, long long total_tasks, hipStream_t stream,
-                                    const uint64_t* d_tbl, const int32_t* d_slot_map, const Dims& d, int slabs) {
-    if (total_tasks <= 0) return hipSuccess;
-    if (total_tasks > 0x7fffffffll) return hipErrorInvalidValue;
-    const int blocks = (int)((total_tasks + waves_per_block - 1) / waves_per_block);
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(waves_per_block * 64), 0, stream, d_tbl, d_slot_map, d.R, d.E, d.K,
-                       d.max_tokens, d.H, slabs, d.Tgrid, (int)total_tasks);
+    auto kern = use_fp8 ? layout_kernel<true> : layout_kernel<false>;
+    if (lds > 48 * 1024) {
+        hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+    }
+    hipLaunchKernelGGL(kern, dim3(d.E), dim3(block), lds, stream, d_tbl, d_routes, stamp, d.R, d.E, d.K, d.H,
+                       d.max_tokens, words_per_rank, t.layout_rotate);
     return hipGetLastError();
 }
 
 static int clamp_waves(int w) { return w < 1 ? 1 : (w > 8 ? 8 : w); }
 
-hipError_t launch_pack(const uint64_t* d_tbl, const int32_t* d_slot_map, float* /*d_scale_stage*/, const Dims& d,
-                       bool use_fp8, const Tuning& t, hipStream_t stream) {
+template <typename Kern>
+static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp,
+                                const PackLaunch& pl, float* stage, const Dims& d, const Tuning& t,
+                                hipStream_t stream) {
     const int slabs = (d.H + 1023) / 1024;
     const long long total = (long long)d.R * d.Tgrid * slabs;
+    if (total <= 0) return hipSuccess;
+    if (total > 0x7fffffffll) return hipErrorInvalidValue;
     const int wpb = clamp_waves(t.pack_waves);
-    const bool ntl = t.nontemporal & 1, nts = t.nontemporal & 2;
-#define MCEP_PACK(KERN)                                                                                      \
-    (ntl ? (nts ? launch_wave_tasks(KERN<true, true>, wpb, total, stream, d_tbl, d_slot_map, d, slabs)       \
-                : launch_wave_tasks(KERN<true, false>, wpb, total, stream, d_tbl, d_slot_map, d, slabs))     \
-         : (nts ? launch_wave_tasks(KERN<false, true>, wpb, total, stream, d_tbl, d_slot_map, d, slabs)      \
-                : launch_wave_tasks(KERN<false, false>, wpb, total, stream, d_tbl, d_slot_map, d, slabs)))
-    if (!use_fp8) return MCEP_PACK(pack_bf16_kernel);
-    if (t.pack_variant == 1) return MCEP_PACK(pack_fp8_split_kernel);
-    return MCEP_PACK(pack_fp8_kernel);
-#undef MCEP_PACK
+    const int blocks = (int)((total + wpb - 1) / wpb);
+    PackSource src;
+    src.x_base = pl.x_base;
+    src.x_stride = pl.x_stride;
+    src.tokens = pl.uniform_tokens;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_routes, stamp, src, stage, d.R, d.K,
+                       d.max_tokens, d.H, slabs, d.Tgrid, (int)total);
+    return hipGetLastError();
 }
 
-hipError_t launch_resolve(const uint64_t* d_tbl, int32_t* d_slot_map, const Dims& d, const Tuning& /*t*/,
-                          hipStream_t stream) {
-    const long long total = (long long)d.R * d.Tgrid;
+hipError_t launch_pack(const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp, const PackLaunch& pl,
+                       const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream) {
+    const bool ntl = t.pack_nt & 1, nts = t.pack_nt & 2;
+    float* stage = (use_fp8 && t.scale_mode == 1) ? pl.scale_stage : nullptr;
+#define MCEP_PACK(KERN)                                                                                \
+    (ntl ? (nts ? launch_pack_t(KERN<true, true>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)     \
+                : launch_pack_t(KERN<true, false>, d_tbl, d_routes, stamp, pl, stage, d, t, stream))   \
+         : (nts ? launch_pack_t(KERN<false, true>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)    \
+                : launch_pack_t(KERN<false, false>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)))
+    hipError_t err;
+    if (!use_fp8) err = MCEP_PACK(pack_bf16_kernel);
+    else if (t.pack_variant == 1) err = MCEP_PACK(pack_fp8_split_kernel);
+    else err = MCEP_PACK(pack_fp8_kernel);
+#undef MCEP_PACK
+    if (err != hipSuccess || stage == nullptr) return err;
+    const long long total = (long long)d.E * kTransposeWaves;
+    const int wpb = 4;
+    hipLaunchKernelGGL(scale_transpose_kernel, dim3((unsigned)((total + wpb - 1) / wpb)), dim3(wpb * 64), 0, stream,
+                       d_tbl, stage, d.R, d.E, d.H / 128, d.max_tokens, (int)total);
+    return hipGetLastError();
+}
+
+hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, const Dims& d,
+                          const Tuning& /*t*/, hipStream_t stream) {
+    const long long total = (long long)d.E * d.R;
     if (total <= 0) return hipSuccess;
+    if (total > 0x7fffffffll) return hipErrorInvalidValue;
     const int wpb = 4;
     const int blocks = (int)((total + wpb - 1) / wpb);
-    hipLaunchKernelGGL(resolve_kernel, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_slot_map, d.R, d.E, d.K,
-                       d.max_tokens, d.Tgrid, (int)total);
+    hipLaunchKernelGGL(resolve_kernel, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_routes, stamp, d.R, d.E, d.K,
+                       d.H, d.max_tokens, (int)total);
     return hipGetLastError();
 }
 
 template <int KMAX, int CH>
-static hipError_t launch_reduce_t(const uint64_t* d_tbl, const int32_t* d_slot_map, const void* d_zero_row,
-                                  const Dims& d, const Tuning& t, hipStream_t stream) {
+static hipError_t launch_reduce_t(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp,
+                                  const void* d_zero_row, const Dims& d, const Tuning& t, hipStream_t stream) {
     const int slabs = (d.H + CH * 512 - 1) / (CH * 512);
     const long long total = (long long)d.R * d.Tgrid * slabs;
     if (total <= 0) return hipSuccess;
     if (total > 0x7fffffffll) return hipErrorInvalidValue;
     const int wpb = clamp_waves(t.combine_waves);
     const int blocks = (int)((total + wpb - 1) / wpb);
-    const bool ntl = t.nontemporal & 1, nts = t.nontemporal & 2;
+    const bool ntl = t.combine_nt & 1, nts = t.combine_nt & 2;
 #define MCEP_REDUCE(A, B)                                                                                       \
-    hipLaunchKernelGGL((reduce_kernel<KMAX, CH, A, B>), dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_slot_map, \
-                       d_zero_row, d.R, d.E, d.K, d.max_tokens, d.H, slabs, d.Tgrid, (int)total)
+    hipLaunchKernelGGL((reduce_kernel<KMAX, CH, A, B>), dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_routes, \
+                       stamp, d_zero_row, d.R, d.K, d.max_tokens, d.H, slabs, d.Tgrid, (int)total)
     if (ntl && nts) MCEP_REDUCE(true, true);
     else if (ntl) MCEP_REDUCE(true, false);
     else if (nts) MCEP_REDUCE(false, true);
@@ -645,12 +810,12 @@ static hipError_t launch_reduce_t(const uint64_t* d_tbl, const int32_t* d_slot_m
     return hipGetLastError();
 }
 
-hipError_t launch_reduce(const uint64_t* d_tbl, const int32_t* d_slot_map, const void* d_zero_row, const Dims& d,
-                         const Tuning& t, hipStream_t stream) {
+hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const void* d_zero_row,
+                         const Dims& d, const Tuning& t, hipStream_t stream) {
     const int ch = t.combine_chunks >= 2 ? 2 : 1;
-#define MCEP_K(KMAX)                                                                             \
-    return ch == 2 ? launch_reduce_t<KMAX, 2>(d_tbl, d_slot_map, d_zero_row, d, t, stream)       \
-                   : launch_reduce_t<KMAX, 1>(d_tbl, d_slot_map, d_zero_row, d, t, stream)
+#define MCEP_K(KMAX)                                                                                    \
+    return ch == 2 ? launch_reduce_t<KMAX, 2>(d_tbl, d_routes, stamp, d_zero_row, d, t, stream)         \
+                   : launch_reduce_t<KMAX, 1>(d_tbl, d_routes, stamp, d_zero_row, d, t, stream)
     if (d.K <= 1) { MCEP_K(1); }
     if (d.K <= 2) { MCEP_K(2); }
     if (d.K <= 4) { MCEP_K(4); }

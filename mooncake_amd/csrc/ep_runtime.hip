@@ -83,8 +83,11 @@ struct mc_ep_world {
     hipStream_t comm_stream = nullptr;
     uint64_t* d_tbl[2] = {nullptr, nullptr};     // dispatch, combine pointer tables
     std::vector<uint64_t> tbl_cache[2];           // what the device tables hold
-    int32_t* d_slot[2] = {nullptr, nullptr};     // (rank, token, k) -> packed row
-    size_t slot_cap[2] = {0, 0};
+    void* d_routes[2] = {nullptr, nullptr};      // per-selection routes: DispatchRoute[], CombineRoute[]
+    size_t route_cap[2] = {0, 0};                 // capacity in selections
+    uint32_t stamp[2] = {0, 0};                   // launch counter the routes are stamped with
+    float* d_scale_stage = nullptr;               // fp8 scales of each token before transposition
+    size_t scale_stage_cap = 0;                   // capacity in floats
     void* d_zero_row = nullptr;
     Tuning tuning;
     std::vector<char> silent;
@@ -125,16 +128,32 @@ struct DeviceGuard {
     }
 };
 
-int ensure_slot_map(mc_ep_world* w, int which, size_t words) {
-    if (words <= w->slot_cap[which]) return MC_EP_OK;
-    // grows only; the old map may still be read by queued kernels
+int ensure_routes(mc_ep_world* w, int which, size_t selections) {
+    if (selections <= w->route_cap[which]) return MC_EP_OK;
+    // grows only; the old table may still be read by queued kernels
     MC_HIP(hipDeviceSynchronize());
-    if (w->d_slot[which]) MC_HIP(hipFree(w->d_slot[which]));
-    w->d_slot[which] = nullptr;
-    w->slot_cap[which] = 0;
-    size_t cap = words + words / 2 + 1024;
-    MC_HIP(hipMalloc((void**)&w->d_slot[which], cap * sizeof(int32_t)));
-    w->slot_cap[which] = cap;
+    if (w->d_routes[which]) MC_HIP(hipFree(w->d_routes[which]));
+    w->d_routes[which] = nullptr;
+    w->route_cap[which] = 0;
+    const size_t cap = selections + selections / 2 + 1024;
+    const size_t bytes = cap * (which == 0 ? sizeof(DispatchRoute) : sizeof(CombineRoute));
+    MC_HIP(hipMalloc(&w->d_routes[which], bytes));
+    // stamps start at 1, so a zeroed table holds no valid route
+    MC_HIP(hipMemset(w->d_routes[which], 0, bytes));
+    w->stamp[which] = 0;
+    w->route_cap[which] = cap;
+    return MC_EP_OK;
+}
+
+int ensure_scale_stage(mc_ep_world* w, size_t floats) {
+    if (floats <= w->scale_stage_cap) return MC_EP_OK;
+    MC_HIP(hipDeviceSynchronize());
+    if (w->d_scale_stage) MC_HIP(hipFree(w->d_scale_stage));
+    w->d_scale_stage = nullptr;
+    w->scale_stage_cap = 0;
+    const size_t cap = floats + floats / 2 + 1024;
+    MC_HIP(hipMalloc((void**)&w->d_scale_stage, cap * sizeof(float)));
+    w->scale_stage_cap = cap;
     return MC_EP_OK;
 }
 
@@ -188,12 +207,34 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         if (num_tokens[r] > tgrid) tgrid = num_tokens[r];
     }
     DeviceGuard guard(w->device);
-    if (int rc = ensure_slot_map(w, 0, (size_t)R * max_tokens * num_topk)) return rc;
-    if (int rc = upload_table(w, 0, tbl, stream)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
-    if (phases & MC_EP_PHASE_LAYOUT) MC_HIP(launch_layout(w->d_tbl[0], w->d_slot[0], d, w->tuning, stream));
-    if ((phases & MC_EP_PHASE_DATA) && tgrid > 0)
-        MC_HIP(launch_pack(w->d_tbl[0], w->d_slot[0], nullptr, d, use_fp8 != 0, w->tuning, stream));
+    // the layout kernel keeps one ballot per 64 selections of the world in LDS
+    MC_ASSERT(layout_lds_bytes(d) <= kMaxLayoutLdsBytes);
+    if (int rc = ensure_routes(w, 0, (size_t)R * max_tokens * num_topk)) return rc;
+    if (int rc = upload_table(w, 0, tbl, stream)) return rc;
+    auto* routes = (DispatchRoute*)w->d_routes[0];
+    if (phases & MC_EP_PHASE_LAYOUT) {
+        w->stamp[0] += 1;
+        MC_HIP(launch_layout(w->d_tbl[0], routes, w->stamp[0], d, use_fp8 != 0, w->tuning, stream));
+    }
+    if ((phases & MC_EP_PHASE_DATA) && tgrid > 0) {
+        PackLaunch pl;
+        if (use_fp8 && w->tuning.scale_mode == 1) {
+            if (int rc = ensure_scale_stage(w, (size_t)R * max_tokens * (hidden / 128))) return rc;
+            pl.scale_stage = w->d_scale_stage;
+        }
+        // evenly spaced x tensors with one token count: addresses from kernel arguments
+        bool uniform = w->tuning.pack_uniform != 0 && x[0] != 0;
+        const int64_t stride = R > 1 ? (int64_t)(x[1] - x[0]) : 0;
+        for (int r = 0; r < R && uniform; ++r)
+            uniform = num_tokens[r] == num_tokens[0] && x[r] == x[0] + (uint64_t)(stride * r);
+        if (uniform) {
+            pl.x_base = x[0];
+            pl.x_stride = stride;
+            pl.uniform_tokens = num_tokens[0];
+        }
+        MC_HIP(launch_pack(w->d_tbl[0], routes, w->stamp[0], pl, d, use_fp8 != 0, w->tuning, stream));
+    }
     return MC_EP_OK;
 }
 
@@ -227,12 +268,16 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     }
     if (tgrid == 0) return MC_EP_OK;
     DeviceGuard guard(w->device);
-    if (int rc = ensure_slot_map(w, 1, (size_t)R * max_tokens * num_topk)) return rc;
+    if (int rc = ensure_routes(w, 1, (size_t)R * max_tokens * num_topk)) return rc;
     if (int rc = upload_table(w, 1, tbl, stream)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
-    if (phases & MC_EP_PHASE_LAYOUT) MC_HIP(launch_resolve(w->d_tbl[1], w->d_slot[1], d, w->tuning, stream));
+    auto* routes = (CombineRoute*)w->d_routes[1];
+    if (phases & MC_EP_PHASE_LAYOUT) {
+        w->stamp[1] += 1;
+        MC_HIP(launch_resolve(w->d_tbl[1], routes, w->stamp[1], d, w->tuning, stream));
+    }
     if (phases & MC_EP_PHASE_DATA)
-        MC_HIP(launch_reduce(w->d_tbl[1], w->d_slot[1], w->d_zero_row, d, w->tuning, stream));
+        MC_HIP(launch_reduce(w->d_tbl[1], routes, w->stamp[1], w->d_zero_row, d, w->tuning, stream));
     return MC_EP_OK;
 }
 
@@ -468,9 +513,10 @@ int mc_ep_world_destroy(mc_ep_world_t* w) {
     (void)hipDeviceSynchronize();
     for (int i = 0; i < 2; ++i) {
         if (w->d_tbl[i]) (void)hipFree(w->d_tbl[i]);
-        if (w->d_slot[i]) (void)hipFree(w->d_slot[i]);
+        if (w->d_routes[i]) (void)hipFree(w->d_routes[i]);
     }
     if (w->d_zero_row) (void)hipFree(w->d_zero_row);
+    if (w->d_scale_stage) (void)hipFree(w->d_scale_stage);
     if (w->comm_stream) (void)hipStreamDestroy(w->comm_stream);
     delete w;
     return MC_EP_OK;
@@ -488,12 +534,15 @@ int mc_ep_world_set_rank_silent(mc_ep_world_t* w, int rank, int silent) {
 
 static int* option_slot(Tuning& t, const char* name) {
     if (!strcmp(name, "layout_block")) return &t.layout_block;
+    if (!strcmp(name, "layout_rotate")) return &t.layout_rotate;
     if (!strcmp(name, "pack_variant")) return &t.pack_variant;
     if (!strcmp(name, "pack_waves")) return &t.pack_waves;
     if (!strcmp(name, "scale_mode")) return &t.scale_mode;
     if (!strcmp(name, "combine_chunks")) return &t.combine_chunks;
     if (!strcmp(name, "combine_waves")) return &t.combine_waves;
-    if (!strcmp(name, "nontemporal")) return &t.nontemporal;
+    if (!strcmp(name, "pack_nt")) return &t.pack_nt;
+    if (!strcmp(name, "pack_uniform")) return &t.pack_uniform;
+    if (!strcmp(name, "combine_nt")) return &t.combine_nt;
     return nullptr;
 }
 

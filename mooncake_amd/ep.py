@@ -56,25 +56,53 @@ class World:
         _lib.check(_lib.lib().mc_ep_world_get_option(self._h, name.encode(), ctypes.byref(out)))
         return out.value
 
-    # whole-world calls: every rank's tensors in one launch sequence
+    # whole-world calls: every rank's tensors in one launch sequence.  The
+    # prepare_* forms marshal the per-rank pointer arrays once and return a
+    # callable (stream_ptr, phases) for callers that repeat the same call.
+    def prepare_dispatch(self, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk,
+                         num_max_dispatch_tokens_per_rank, num_experts, use_fp8, recv_x_ptrs, recv_scales_ptrs,
+                         recv_count_ptrs, src_info_ptrs, layout_range_ptrs):
+        u = _lib.u64_array
+        fn = _lib.lib().mc_ep_world_dispatch
+        args = (self._h, u(x_ptrs), u(topk_idx_ptrs), _lib.i32_array(num_tokens), hidden, num_topk,
+                num_max_dispatch_tokens_per_rank, num_experts, int(bool(use_fp8)), u(recv_x_ptrs),
+                u(recv_scales_ptrs) if recv_scales_ptrs is not None else None, u(recv_count_ptrs),
+                u(src_info_ptrs), u(layout_range_ptrs))
+
+        def call(stream_ptr: int, phases: int = _lib.PHASE_ALL) -> None:
+            rc = fn(*args, phases, stream_ptr)
+            if rc:
+                _lib.check(rc)
+        return call
+
+    def prepare_combine(self, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
+                        active_ranks_ptrs, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
+                        num_experts, combined_x_ptrs):
+        u = _lib.u64_array
+        fn = _lib.lib().mc_ep_world_combine
+        args = (self._h, u(x_ptrs), u(topk_idx_ptrs), u(topk_weights_ptrs), u(src_info_ptrs), u(layout_range_ptrs),
+                u(active_ranks_ptrs), _lib.i32_array(num_combined_tokens), hidden, num_topk,
+                num_max_dispatch_tokens_per_rank, num_experts, u(combined_x_ptrs))
+
+        def call(stream_ptr: int, phases: int = _lib.PHASE_ALL) -> None:
+            rc = fn(*args, phases, stream_ptr)
+            if rc:
+                _lib.check(rc)
+        return call
+
     def dispatch(self, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
                  num_experts, use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
                  layout_range_ptrs, stream_ptr: int, phases: int = _lib.PHASE_ALL) -> None:
-        u = _lib.u64_array
-        scales = u(recv_scales_ptrs) if recv_scales_ptrs is not None else None
-        _lib.check(_lib.lib().mc_ep_world_dispatch(
-            self._h, u(x_ptrs), u(topk_idx_ptrs), _lib.i32_array(num_tokens), hidden, num_topk,
-            num_max_dispatch_tokens_per_rank, num_experts, int(bool(use_fp8)), u(recv_x_ptrs), scales,
-            u(recv_count_ptrs), u(src_info_ptrs), u(layout_range_ptrs), phases, stream_ptr))
+        self.prepare_dispatch(x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
+                              num_experts, use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
+                              layout_range_ptrs)(stream_ptr, phases)
 
     def combine(self, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
                 active_ranks_ptrs, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
                 num_experts, combined_x_ptrs, stream_ptr: int, phases: int = _lib.PHASE_ALL) -> None:
-        u = _lib.u64_array
-        _lib.check(_lib.lib().mc_ep_world_combine(
-            self._h, u(x_ptrs), u(topk_idx_ptrs), u(topk_weights_ptrs), u(src_info_ptrs), u(layout_range_ptrs),
-            u(active_ranks_ptrs), _lib.i32_array(num_combined_tokens), hidden, num_topk,
-            num_max_dispatch_tokens_per_rank, num_experts, u(combined_x_ptrs), phases, stream_ptr))
+        self.prepare_combine(x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
+                             active_ranks_ptrs, num_combined_tokens, hidden, num_topk,
+                             num_max_dispatch_tokens_per_rank, num_experts, combined_x_ptrs)(stream_ptr, phases)
 
 
 _default_worlds: Dict[int, World] = {}

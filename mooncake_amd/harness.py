@@ -29,6 +29,7 @@ class WorldHarness:
         self.recv_x = self.recv_scales_phys = self.recv_count = self.src_info = self.layout_range = None
         self.expert_out = self.combined = None
         self.active_ranks = torch.ones((R, R), dtype=torch.int32, device=self.device)
+        self._prepared = {}     # marshalled whole-world calls, keyed by (kind, present)
 
     # ------------------------------------------------------------------
     def load(self, data: Dict[str, torch.Tensor]) -> None:
@@ -80,24 +81,35 @@ class WorldHarness:
         """present[r] == 0 makes rank r silent: it neither sends nor receives."""
         c = self.cfg
         R = c.num_ranks
-        nt = [n if (present is None or present[r]) else 0 for r, n in enumerate(self.num_tokens)]
-        self.world.dispatch(
-            self._ptrs(self.x, R), self._ptrs(self.topk_idx, R), nt, c.hidden, c.num_topk, c.max_tokens,
-            c.num_experts, c.use_fp8, self._ptrs(self.recv_x, R, present),
-            self._ptrs(self.recv_scales_phys, R, present) if c.use_fp8 else None,
-            self._ptrs(self.recv_count, R, present), self._ptrs(self.src_info, R, present),
-            self._ptrs(self.layout_range, R, present), self._stream(stream), phases)
+        key = ("dispatch", None if present is None else tuple(present), self.x.data_ptr(), self.recv_x.data_ptr())
+        call = self._prepared.get(key)
+        if call is None:
+            nt = [n if (present is None or present[r]) else 0 for r, n in enumerate(self.num_tokens)]
+            call = self.world.prepare_dispatch(
+                self._ptrs(self.x, R), self._ptrs(self.topk_idx, R), nt, c.hidden, c.num_topk, c.max_tokens,
+                c.num_experts, c.use_fp8, self._ptrs(self.recv_x, R, present),
+                self._ptrs(self.recv_scales_phys, R, present) if c.use_fp8 else None,
+                self._ptrs(self.recv_count, R, present), self._ptrs(self.src_info, R, present),
+                self._ptrs(self.layout_range, R, present))
+            self._prepared[key] = call
+        call(self._stream(stream), phases)
 
     def combine(self, phases: int = _lib.PHASE_ALL, stream: Optional[torch.cuda.Stream] = None,
                 present: Optional[Sequence[int]] = None) -> None:
         c = self.cfg
         R = c.num_ranks
-        nt = [n if (present is None or present[r]) else 0 for r, n in enumerate(self.num_tokens)]
-        self.world.combine(
-            self._ptrs(self.expert_out, R, present), self._ptrs(self.topk_idx, R), self._ptrs(self.topk_weights, R),
-            self._ptrs(self.src_info, R), self._ptrs(self.layout_range, R), self._ptrs(self.active_ranks, R), nt,
-            c.hidden, c.num_topk, c.max_tokens, c.num_experts, self._ptrs(self.combined, R), self._stream(stream),
-            phases)
+        key = ("combine", None if present is None else tuple(present), self.expert_out.data_ptr(),
+               self.combined.data_ptr(), self.src_info.data_ptr())
+        call = self._prepared.get(key)
+        if call is None:
+            nt = [n if (present is None or present[r]) else 0 for r, n in enumerate(self.num_tokens)]
+            call = self.world.prepare_combine(
+                self._ptrs(self.expert_out, R, present), self._ptrs(self.topk_idx, R),
+                self._ptrs(self.topk_weights, R), self._ptrs(self.src_info, R), self._ptrs(self.layout_range, R),
+                self._ptrs(self.active_ranks, R), nt, c.hidden, c.num_topk, c.max_tokens, c.num_experts,
+                self._ptrs(self.combined, R))
+            self._prepared[key] = call
+        call(self._stream(stream), phases)
 
     # ------------------------------------------------------------------
     def recv_x_typed(self) -> torch.Tensor:

@@ -153,14 +153,12 @@ ORACLE_API void oracle_quantise_rows(const uint16_t* x, int64_t rows, int H, uin
 /* routing layout                                                            */
 /* ------------------------------------------------------------------------ */
 
-static inline int token_selects(const int64_t* row, int K, int64_t e) {
-    for (int k = 0; k < K; ++k) if (row[k] == e) return 1;   /* `.any(dim=1)`, PY:797-802 */
-    return 0;
-}
-
 /* Order and ranges as PY:787-817: for each local expert, source ranks in
- * ascending order, within a rank tokens in ascending order (a token counts
- * once even if it names the expert twice); layout_range = (begin << 32) |
+ * ascending order, within a rank tokens in ascending order.  The contract has
+ * a token name an expert at most once; should it name one twice, each
+ * occurrence gets its own row in k order, as the kernel sends once per k
+ * (K:230, K:273) - PY:797-802 would count such a token once.
+ * layout_range = (begin << 32) |
  * count with count in the low half (U:160-169, PY:1023-1024) and 0 for an
  * empty pair (PY:817); src_info[row] = token index at the source (K:231,
  * K:446, PY:838).  recv_count = sum of counts (K:430, PY:831).  Rows at and
@@ -183,13 +181,14 @@ ORACLE_API void oracle_layout(int R, int E, int K, int Tmax, int max_tokens, con
             const int T = (src_present && !src_present[r]) ? 0 : num_tokens[r];
             for (int t = 0; t < T; ++t) {
                 const int64_t* row = topk_idx + ((int64_t)r * Tmax + t) * K;
-                if (!token_selects(row, K, e)) continue;
-                const int slot = begin + count;
-                src_info[((int64_t)q * L + le) * RM + slot] = t;
-                if (slot_map)
-                    for (int k = 0; k < K; ++k)
-                        if (row[k] == e) slot_map[((int64_t)r * Tmax + t) * K + k] = slot;
-                ++count;
+                for (int k = 0; k < K; ++k) {
+                    if (row[k] != e) continue;
+                    if ((int64_t)begin + count >= RM) continue;   /* only duplicates can overflow: dropped */
+                    const int slot = begin + count;
+                    src_info[((int64_t)q * L + le) * RM + slot] = t;
+                    if (slot_map) slot_map[((int64_t)r * Tmax + t) * K + k] = slot;
+                    ++count;
+                }
             }
             layout_range[((int64_t)q * L + le) * R + r] = count ? (((int64_t)begin << 32) | (int64_t)count) : 0;
             begin += count;
@@ -230,10 +229,6 @@ ORACLE_API void oracle_dispatch(int R, int E, int K, int Tmax, int max_tokens, i
                 const int64_t e = topk_idx[n * K + k];
                 const int slot = slot_map[n * K + k];
                 if (e < 0 || slot < 0) continue;
-                /* a duplicated expert maps to one shared row: written once */
-                int dup = 0;
-                for (int k2 = 0; k2 < k; ++k2) dup |= (topk_idx[n * K + k2] == e);
-                if (dup) continue;
                 const int64_t row = (int64_t)e * RM + slot;   /* == (q*L + le)*RM + slot */
                 if (use_fp8) {
                     memcpy((uint8_t*)recv_x + row * H, qrow, (size_t)H);

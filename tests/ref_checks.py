@@ -24,8 +24,9 @@ def brute_force_layout(topk_idx: torch.Tensor, num_tokens: Sequence[int], max_to
         if src_present is not None and not src_present[r]:
             continue
         for t in range(num_tokens[r]):
-            for e in sorted(set(v for v in idx[r][t] if v >= 0)):
-                per_expert[e].append((r, t))
+            for e in idx[r][t]:                # one row per (token, k) occurrence, in k order
+                if e >= 0:
+                    per_expert[e].append((r, t))
     out = {"recv_count": [[0] * L for _ in range(R)],
            "layout_range": [[[0] * R for _ in range(L)] for _ in range(R)],
            "src_info": [[[] for _ in range(L)] for _ in range(R)],

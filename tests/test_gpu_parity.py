@@ -43,12 +43,29 @@ def test_dispatch_matches_oracle(gpu_device, oracle, cfg, is_ragged):
 
 
 @pytest.mark.parametrize("variant", [0, 1])
-@pytest.mark.parametrize("nontemporal", [0, 3])
-def test_fp8_pack_variants_match_oracle(gpu_device, oracle, variant, nontemporal):
+@pytest.mark.parametrize("nt", [0, 3])
+@pytest.mark.parametrize("scale_mode", [0, 1])
+@pytest.mark.parametrize("uniform", [0, 1])
+def test_fp8_pack_variants_match_oracle(gpu_device, oracle, variant, nt, scale_mode, uniform):
+    """Every tuning variant of the pack path is the same function."""
     cfg = EPConfig("variants", 4, 24, 2560, 16, 3, True)
-    announce(f"pack variant={variant} nontemporal={nontemporal}")
+    announce(f"pack variant={variant} nt={nt} scale_mode={scale_mode} uniform={uniform}")
     data = generate(cfg, seed=1)
-    h = run_dispatch(cfg, data, poison=True, options={"pack_variant": variant, "nontemporal": nontemporal})
+    h = run_dispatch(cfg, data, poison=True, options={"pack_variant": variant, "pack_nt": nt,
+                                                      "scale_mode": scale_mode, "pack_uniform": uniform})
+    ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, True)
+    compare_dispatch(h, ref, check_poison=True)
+
+
+@pytest.mark.parametrize("opts", [{"layout_rotate": 0}, {"layout_block": 256}, {"layout_block": 64},
+                                  {"pack_waves": 1}, {"pack_waves": 8}, {"pack_nt": 1}, {"pack_nt": 2}],
+                         ids=lambda o: "-".join(f"{k}{v}" for k, v in o.items()))
+def test_dispatch_tuning_options_match_oracle(gpu_device, oracle, opts):
+    cfg = EPConfig("opts", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05)
+    announce(f"dispatch options {opts}")
+    data = generate(cfg, seed=2)
+    nt = ragged(cfg, True)
+    h = run_dispatch(cfg, data, num_tokens=nt, poison=True, options=opts)
     ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, True)
     compare_dispatch(h, ref, check_poison=True)
 
@@ -107,6 +124,20 @@ def test_fp8_inf_and_nan_inputs(gpu_device, oracle):
                        ref["scales"][0, 0, :T].contiguous().view(torch.int32))
 
 
+def test_duplicate_experts_follow_the_oracle(gpu_device, oracle):
+    """Out of contract, but defined: one row per (token, k) occurrence; rows that
+    would overflow a block's capacity are dropped."""
+    cfg = EPConfig("dups", 2, 16, 1024, 4, 4, True)
+    announce("dispatch with repeated experts in a token")
+    data = generate(cfg, seed=6)
+    data["topk_idx"][:, ::3, 1] = data["topk_idx"][:, ::3, 0]          # k=1 repeats k=0 on every third token
+    data["topk_idx"][0, :, :] = 1                                      # rank 0: every token names expert 1 four times
+    h = run_dispatch(cfg, data, poison=True)
+    ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, True)
+    assert int(ref["recv_count"].max()) == cfg.num_ranks * cfg.max_tokens   # the overflow case is exercised
+    compare_dispatch(h, ref, check_poison=True)
+
+
 COMBINE_CASES = [
     EPConfig("tiny_c", 2, 4, 128, 4, 2, False),
     EPConfig("odd_hidden_c", 4, 24, 2560, 16, 3, False),
@@ -120,12 +151,12 @@ COMBINE_CASES = [
 
 @pytest.mark.parametrize("cfg", COMBINE_CASES, ids=[c.name for c in COMBINE_CASES])
 @pytest.mark.parametrize("is_ragged", [False, True], ids=["full", "ragged"])
-@pytest.mark.parametrize("chunks", [1, 2])
-def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks):
+@pytest.mark.parametrize("chunks,cnt", [(1, 3), (2, 3), (1, 0)])
+def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks, cnt):
     nt = ragged(cfg, is_ragged)
-    announce(f"combine {cfg} ragged={nt} chunks={chunks}")
+    announce(f"combine {cfg} ragged={nt} chunks={chunks} nt={cnt}")
     data = generate(cfg, seed=3)
-    h = run_dispatch(cfg, data, num_tokens=nt, poison=False, options={"combine_chunks": chunks})
+    h = run_dispatch(cfg, data, num_tokens=nt, poison=False, options={"combine_chunks": chunks, "combine_nt": cnt})
     factor = torch.arange(cfg.num_experts).float() * 0.1 + 1.0
     h.alloc_combine_io()
     h.expert_out.fill_(float("nan"))                       # rows outside the handle must never be read

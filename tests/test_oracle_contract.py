@@ -74,11 +74,18 @@ def test_silent_source_rank_sends_nothing(oracle):
     assert bool((got["layout_range"][:, :, 1] == 0).all())
 
 
-def test_duplicate_expert_counts_once(oracle):
+def test_duplicate_expert_gets_a_row_per_occurrence(oracle):
+    # out of contract (every workload picks distinct experts); pinned to the kernel's behaviour:
+    # one send per k (mooncake_ep_kernel.cu:230,273)
     idx = torch.tensor([[[1, 1], [0, 1]]], dtype=torch.int64)
+    got = oracle.layout(idx, [2], 4, 2)
+    assert got["recv_count"].tolist() == [[1, 3]]
+    assert got["slot_map"].tolist() == [[[0, 1], [0, 2]]]
+    assert got["src_info"][0, 1, :3].tolist() == [0, 0, 1]
+    # more duplicate rows than the block can hold: the excess is dropped, counts saturate at capacity
     got = oracle.layout(idx, [2], 2, 2)
     assert got["recv_count"].tolist() == [[1, 2]]
-    assert got["slot_map"].tolist() == [[[0, 0], [0, 1]]]
+    assert got["slot_map"].tolist() == [[[0, 1], [0, -1]]]
 
 
 @pytest.mark.parametrize("use_fp8", [False, True])
