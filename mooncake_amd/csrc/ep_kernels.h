@@ -75,7 +75,7 @@ struct Tuning {
     int layout_rotate = 1;     // start each expert block at its own offset into the selection list
     int pack_variant = 0;      // 0: 32 B/lane loads, 16 B stores; 1: two coalesced 16 B loads, 8 B stores
     int pack_waves = 4;        // waves per block in the pack kernel
-    int pack_nt = 3;           // bit 0: streaming (nontemporal) loads, bit 1: streaming stores
+    int pack_nt = 1;           // bit 0: streaming (nontemporal) loads, bit 1: streaming stores
     int pack_uniform = 1;      // take x addresses from kernel arguments when the ranks' x are evenly spaced
     int scale_mode = 1;        // 0: scatter scales from the pack kernel; 1: staged + transposing pass
     int combine_chunks = 1;    // 16-byte chunks per lane in the combine kernel
@@ -89,12 +89,14 @@ struct PackLaunch {
     int64_t x_stride = 0;
     int uniform_tokens = 0;
     float* scale_stage = nullptr;   // [R * max_tokens, H / 128] staging rows for fp8 scales
+    int32_t* row_src = nullptr;     // [E, R * max_tokens] packed row -> source token slot, from the layout kernel
+    int32_t* counts = nullptr;      // [E] rows per expert, from the layout kernel
 };
 
 hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_words, hipStream_t stream);
 
-hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, uint32_t stamp, const Dims& d, bool use_fp8,
-                         const Tuning& t, hipStream_t stream);
+hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, int32_t* d_row_src, int32_t* d_counts,
+                         uint32_t stamp, const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream);
 hipError_t launch_pack(const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp, const PackLaunch& pl,
                        const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream);
 hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, const Dims& d,

@@ -112,16 +112,23 @@ __global__ void table_write_kernel(uint64_t* dst, TableChunk chunk, int n) {
 //   scan    exclusive prefix of the per-word popcounts = packed row of the
 //           first hit of each word; rank boundaries give (begin, count).
 //   pass 2  ballot bits -> src_info entries and resolved destination routes.
+struct LayoutScratch {
+    int32_t* row_src;    // [E, R*max]  packed row -> source token slot (rank * max_tokens + token)
+    int32_t* counts;     // [E]         recv_count of every global expert
+};
+
 template <bool FP8>
 __global__ __launch_bounds__(1024) void layout_kernel(const uint64_t* __restrict__ tbl,
-                                                       DispatchRoute* __restrict__ routes, uint32_t stamp, int R,
-                                                       int E, int K, int H, int max_tokens, int words_per_rank,
-                                                       int rotate) {
+                                                       DispatchRoute* __restrict__ routes, LayoutScratch scratch,
+                                                       uint32_t stamp, int R, int E, int K, int H, int max_tokens,
+                                                       int words_per_rank, int rotate) {
     extern __shared__ unsigned long long lds[];
     const int W = R * words_per_rank;
-    unsigned long long* masks = lds;                       // [W]
-    int* wbeg = (int*)(lds + W);                           // [W + 1]
-    int* wave_tot = wbeg + W + 1;                          // [16]
+    unsigned long long* masks = lds;                       // [W]   ballots
+    unsigned long long* rank_idx = lds + W;                // [R]   topk_idx address of each rank
+    int* wbeg = (int*)(rank_idx + R);                      // [W+1] packed row of each word's first hit
+    int* rank_n = wbeg + W + 1;                            // [R]   selections (tokens * K) of each rank
+    int* wave_tot = rank_n + R;                            // [16]
 
     const int e = blockIdx.x;
     const int L = E / R, q = e / L, le = e - q * L;
@@ -133,34 +140,60 @@ __global__ __launch_bounds__(1024) void layout_kernel(const uint64_t* __restrict
     // a rank that takes no part in this dispatch receives nothing; routes
     // towards it keep an old stamp and are skipped by the pack kernel
     const uint64_t recv_x = tbl[DF_RECV_X * R + q];
-    if (recv_x == 0) return;
+    if (recv_x == 0) {
+        if (threadIdx.x == 0) scratch.counts[e] = 0;
+        return;
+    }
+    // the rank table is read once per block, not once per word
+    for (int r = threadIdx.x; r < R; r += blockDim.x) {
+        rank_n[r] = (int)tbl[DF_NUM_TOKENS * R + r] * K;
+        rank_idx[r] = tbl[DF_TOPK_IDX * R + r];
+    }
     int32_t* recv_count = (int32_t*)tbl[DF_RECV_COUNT * R + q];
     int32_t* src_info = (int32_t*)tbl[DF_SRC_INFO * R + q] + (int64_t)le * RM;
     int64_t* layout_range = (int64_t*)tbl[DF_LAYOUT_RANGE * R + q] + (int64_t)le * R;
+    __syncthreads();
 
-    // An item is a run of up to U consecutive words of one rank: one rank-table
-    // lookup and one division per item, U independent loads in flight per lane.
-    constexpr int U = 8;
+    // An item is a run of up to U consecutive words of one rank; a wave takes
+    // IPR items per round and has all their loads in flight before the first ballot.
+    constexpr int U = 8, IPR = 4;
     const int items_per_rank = (words_per_rank + U - 1) / U;
     const int items = R * items_per_rank;
     const int start = rotate ? (int)(((long long)e * items) / E) : 0;
-    for (int it = wave; it < items; it += nwaves) {
-        int item = it + start;
-        if (item >= items) item -= items;
-        const int r = item / items_per_rank, w0 = (item - r * items_per_rank) * U;
-        const int n = (int)tbl[DF_NUM_TOKENS * R + r] * K;
-        const int64_t* idx = (const int64_t*)tbl[DF_TOPK_IDX * R + r];
-        int64_t v[U];
+    for (int it0 = wave * IPR; it0 < items; it0 += nwaves * IPR) {
+        int64_t v[IPR][U];
+        int word0[IPR];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int i = (w0 + u) * 64 + lane;
-            v[u] = (w0 + u < words_per_rank && i < n) ? idx[i] : -1;
+        for (int a = 0; a < IPR; ++a) {
+            word0[a] = -1;
+            int item = it0 + a;
+            if (item < items) {
+                item += start;
+                if (item >= items) item -= items;
+                const int r = item / items_per_rank, w0 = (item - r * items_per_rank) * U;
+                const int n = rank_n[r];
+                const int64_t* idx = (const int64_t*)rank_idx[r];
+                word0[a] = r * words_per_rank + w0;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int i = (w0 + u) * 64 + lane;
+                    v[a][u] = (w0 + u < words_per_rank && i < n) ? idx[i] : -1;
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u) v[a][u] = -1;
+            }
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (w0 + u >= words_per_rank) break;
-            const unsigned long long m = __ballot(v[u] == (int64_t)e);
-            if (lane == 0) masks[r * words_per_rank + w0 + u] = m;
+        for (int a = 0; a < IPR; ++a) {
+            if (word0[a] < 0) continue;
+            const int w0 = word0[a] % words_per_rank;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (w0 + u >= words_per_rank) break;
+                const unsigned long long m = __ballot(v[a][u] == (int64_t)e);
+                if (lane == 0) masks[word0[a] + u] = m;
+            }
         }
     }
     __syncthreads();
@@ -191,7 +224,9 @@ __global__ __launch_bounds__(1024) void layout_kernel(const uint64_t* __restrict
     const int cap = (int)(RM < 0x7fffffff ? RM : 0x7fffffff);
     if (threadIdx.x == 0) {
         wbeg[W] = carry;
-        recv_count[le] = carry < cap ? carry : cap;
+        const int kept = carry < cap ? carry : cap;
+        recv_count[le] = kept;
+        scratch.counts[e] = kept;
     }
     __syncthreads();
     for (int r = threadIdx.x; r < R; r += blockDim.x) {
@@ -203,21 +238,31 @@ __global__ __launch_bounds__(1024) void layout_kernel(const uint64_t* __restrict
         layout_range[r] = c ? (((int64_t)b << 32) | (int64_t)c) : 0;
     }
 
+    // Ballot bits -> rows.  32 words per wave step, one per lane; only words
+    // with hits (about one in five for 256 experts) are walked.
     const uint64_t row_bytes = (uint64_t)H * (FP8 ? 1 : 2);
     const uint64_t row0 = recv_x + (uint64_t)le * RM * row_bytes;
     const uint64_t scale0 = FP8 ? tbl[DF_RECV_SCALES * R + q] + (uint64_t)le * (H / 128) * RM * 4 : 0;
-    for (int it = wave; it < items; it += nwaves) {
-        const int r = it / items_per_rank, w0 = (it - r * items_per_rank) * U;
-        for (int u = 0; u < U && w0 + u < words_per_rank; ++u) {
-            const int gi = r * words_per_rank + w0 + u;
-            const unsigned long long m = masks[gi];
-            if (m == 0) continue;
+    int32_t* row_src = scratch.row_src + (int64_t)e * RM;
+    for (int base = wave * 32; base < W; base += nwaves * 32) {
+        const int mine = base + (lane & 31);
+        const unsigned long long mword = (mine < W) ? masks[mine] : 0;
+        const int mbeg = (mine < W) ? wbeg[mine] : 0;
+        unsigned int nz = (unsigned int)__ballot(mword != 0);      // lanes 32..63 mirror lanes 0..31
+        while (nz) {
+            const int j = __builtin_ctz(nz);
+            nz &= nz - 1;
+            const unsigned long long m = read_lane_u64(mword, j);
+            const int wb = __builtin_amdgcn_readlane(mbeg, j);
             if ((m >> lane) & 1ull) {
-                const int pos = wbeg[gi] + __popcll(m & ((1ull << lane) - 1ull));
+                const int pos = wb + __popcll(m & ((1ull << lane) - 1ull));
                 if (pos < cap) {
-                    const int i = (w0 + u) * 64 + lane;
+                    const int gi = base + j;
+                    const int r = gi / words_per_rank, w = gi - r * words_per_rank;
+                    const int i = w * 64 + lane;
                     const int t = i / K, k = i - t * K;
                     src_info[pos] = t;
+                    row_src[pos] = r * max_tokens + t;
                     DispatchRoute rt;
                     rt.row = row0 + (uint64_t)pos * row_bytes;
                     rt.scale = FP8 ? scale0 + (uint64_t)pos * 4 : 0;
@@ -474,45 +519,37 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
 }
 
 // Staged scales -> column-major output.  kTransposeWaves waves per expert,
-// each taking 64 packed rows at a time: a lane finds its row's source token
-// (src_info, and the source rank from the expert's ranges, fetched once per
-// wave), reads that token's H/128 scales as contiguous 16-byte pieces - a
-// batch of them in flight at once - and stores them so that the wave writes
-// 64 consecutive floats per scale group.
+// each taking 64 packed rows at a time: a lane learns its row's source token
+// slot from the layout kernel's row_src, reads that token's H/128 scales as
+// contiguous 16-byte pieces - a batch of them in flight at once - and stores
+// them so that the wave writes 64 consecutive floats per scale group.
 constexpr int kTransposeWaves = 8;
 
 __global__ __launch_bounds__(256) void scale_transpose_kernel(const uint64_t* __restrict__ tbl,
-                                                               const float* __restrict__ scale_stage, int R, int E,
-                                                               int G, int max_tokens, int total_tasks) {
+                                                               const float* __restrict__ scale_stage,
+                                                               LayoutScratch scratch, int R, int E, int G,
+                                                               int max_tokens, int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int e = task / kTransposeWaves, wi = task - e * kTransposeWaves;
     const int L = E / R, q = e / L, le = e - q * L;
-    if (tbl[DF_RECV_X * R + q] == 0) return;
-    const int count = ((const int32_t*)tbl[DF_RECV_COUNT * R + q])[le];
-    if (wi * 64 >= count) return;
     const int64_t RM = (int64_t)R * max_tokens;
-    const int32_t* src_info = (const int32_t*)tbl[DF_SRC_INFO * R + q] + (int64_t)le * RM;
-    const int64_t* ranges = (const int64_t*)tbl[DF_LAYOUT_RANGE * R + q] + (int64_t)le * R;
-    float* out = (float*)tbl[DF_RECV_SCALES * R + q] + (int64_t)le * G * RM;
+    // issued together: the expert's row count, this wave's first source slots
+    // (in bounds whatever the count turns out to be) and the output address
+    const int32_t* row_src = scratch.row_src + (int64_t)e * RM;
+    int row = wi * 64 + lane;
+    int slot = (row < RM) ? row_src[row] : 0;
+    const int count = scratch.counts[e];
+    float* out = (float*)tbl[DF_RECV_SCALES * R + q];
+    if (wi * 64 >= count) return;
+    out += (int64_t)le * G * RM;
 
     for (int row0 = wi * 64; row0 < count; row0 += kTransposeWaves * 64) {
-        const int row = row0 + lane;
+        row = row0 + lane;
         const bool valid = row < count;
-        const int t = valid ? src_info[row] : 0;
-        // source rank of the row: the range that contains it (ranges held one per lane)
-        int r = 0;
-        for (int rb = 0; rb < R; rb += 64) {
-            const int64_t mine = (rb + lane < R) ? ranges[rb + lane] : 0;
-            const int nr = (R - rb < 64) ? (R - rb) : 64;
-            for (int j = 0; j < nr; ++j) {
-                const int c = __builtin_amdgcn_readlane((int)(uint32_t)mine, j);
-                const int b = __builtin_amdgcn_readlane((int)(uint32_t)(mine >> 32), j);
-                if (c != 0 && row >= b && row < b + c) r = rb + j;
-            }
-        }
-        const float* sp = scale_stage + ((int64_t)r * max_tokens + t) * G;
+        if (row0 != wi * 64) slot = valid ? row_src[row] : 0;
+        const float* sp = scale_stage + (int64_t)(valid ? slot : 0) * G;
         float* dp = out + row;
         int g = 0;
         if ((G & 3) == 0) {
@@ -520,7 +557,7 @@ __global__ __launch_bounds__(256) void scale_transpose_kernel(const uint64_t* __
             for (; g + 4 * B <= G; g += 4 * B) {
                 float4 v[B];
 #pragma unroll
-                for (int j = 0; j < B; ++j) v[j] = valid ? *(const float4*)(sp + g + 4 * j) : make_float4(0, 0, 0, 0);
+                for (int j = 0; j < B; ++j) v[j] = *(const float4*)(sp + g + 4 * j);
                 if (valid) {
 #pragma unroll
                     for (int j = 0; j < B; ++j) {
@@ -532,8 +569,8 @@ __global__ __launch_bounds__(256) void scale_transpose_kernel(const uint64_t* __
                 }
             }
             for (; g < G; g += 4) {
+                const float4 v = *(const float4*)(sp + g);
                 if (valid) {
-                    const float4 v = *(const float4*)(sp + g);
                     dp[(int64_t)(g + 0) * RM] = v.x;
                     dp[(int64_t)(g + 1) * RM] = v.y;
                     dp[(int64_t)(g + 2) * RM] = v.z;
@@ -712,11 +749,11 @@ hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_word
 size_t layout_lds_bytes(const Dims& d) {
     const size_t words_per_rank = ((size_t)d.max_tokens * d.K + 63) / 64;
     const size_t W = (size_t)d.R * words_per_rank;
-    return W * 8 + (W + 1) * 4 + 16 * 4 + 16;
+    return W * 8 + (size_t)d.R * 8 + (W + 1) * 4 + (size_t)d.R * 4 + 16 * 4 + 16;
 }
 
-hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, uint32_t stamp, const Dims& d, bool use_fp8,
-                         const Tuning& t, hipStream_t stream) {
+hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, int32_t* d_row_src, int32_t* d_counts,
+                         uint32_t stamp, const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream) {
     const size_t lds = layout_lds_bytes(d);
     if (lds > kMaxLayoutLdsBytes) return hipErrorInvalidValue;
     const int words_per_rank = (int)(((size_t)d.max_tokens * d.K + 63) / 64);
@@ -729,8 +766,9 @@ hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, uint32_
         hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(kern, dim3(d.E), dim3(block), lds, stream, d_tbl, d_routes, stamp, d.R, d.E, d.K, d.H,
-                       d.max_tokens, words_per_rank, t.layout_rotate);
+    LayoutScratch scratch{d_row_src, d_counts};
+    hipLaunchKernelGGL(kern, dim3(d.E), dim3(block), lds, stream, d_tbl, d_routes, scratch, stamp, d.R, d.E, d.K,
+                       d.H, d.max_tokens, words_per_rank, t.layout_rotate);
     return hipGetLastError();
 }
 
@@ -772,8 +810,9 @@ hipError_t launch_pack(const uint64_t* d_tbl, const DispatchRoute* d_routes, uin
     if (err != hipSuccess || stage == nullptr) return err;
     const long long total = (long long)d.E * kTransposeWaves;
     const int wpb = 4;
+    LayoutScratch scratch{pl.row_src, pl.counts};
     hipLaunchKernelGGL(scale_transpose_kernel, dim3((unsigned)((total + wpb - 1) / wpb)), dim3(wpb * 64), 0, stream,
-                       d_tbl, stage, d.R, d.E, d.H / 128, d.max_tokens, (int)total);
+                       d_tbl, stage, scratch, d.R, d.E, d.H / 128, d.max_tokens, (int)total);
     return hipGetLastError();
 }
 

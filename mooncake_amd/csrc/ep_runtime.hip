@@ -86,6 +86,10 @@ struct mc_ep_world {
     void* d_routes[2] = {nullptr, nullptr};      // per-selection routes: DispatchRoute[], CombineRoute[]
     size_t route_cap[2] = {0, 0};                 // capacity in selections
     uint32_t stamp[2] = {0, 0};                   // launch counter the routes are stamped with
+    int32_t* d_row_src = nullptr;                 // [E, R*max] packed row -> source token slot
+    size_t row_src_cap = 0;
+    int32_t* d_counts = nullptr;                  // [E] rows per expert of the last layout
+    size_t counts_cap = 0;
     float* d_scale_stage = nullptr;               // fp8 scales of each token before transposition
     size_t scale_stage_cap = 0;                   // capacity in floats
     void* d_zero_row = nullptr;
@@ -142,6 +146,20 @@ int ensure_routes(mc_ep_world* w, int which, size_t selections) {
     MC_HIP(hipMemset(w->d_routes[which], 0, bytes));
     w->stamp[which] = 0;
     w->route_cap[which] = cap;
+    return MC_EP_OK;
+}
+
+template <typename T>
+int ensure_scratch(T** ptr, size_t* cap, size_t count) {
+    if (count <= *cap) return MC_EP_OK;
+    MC_HIP(hipDeviceSynchronize());
+    if (*ptr) MC_HIP(hipFree(*ptr));
+    *ptr = nullptr;
+    *cap = 0;
+    const size_t grown = count + count / 2 + 1024;
+    MC_HIP(hipMalloc((void**)ptr, grown * sizeof(T)));
+    MC_HIP(hipMemset(*ptr, 0, grown * sizeof(T)));
+    *cap = grown;
     return MC_EP_OK;
 }
 
@@ -211,14 +229,19 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     // the layout kernel keeps one ballot per 64 selections of the world in LDS
     MC_ASSERT(layout_lds_bytes(d) <= kMaxLayoutLdsBytes);
     if (int rc = ensure_routes(w, 0, (size_t)R * max_tokens * num_topk)) return rc;
+    if (int rc = ensure_scratch(&w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
+    if (int rc = ensure_scratch(&w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
     if (int rc = upload_table(w, 0, tbl, stream)) return rc;
     auto* routes = (DispatchRoute*)w->d_routes[0];
     if (phases & MC_EP_PHASE_LAYOUT) {
         w->stamp[0] += 1;
-        MC_HIP(launch_layout(w->d_tbl[0], routes, w->stamp[0], d, use_fp8 != 0, w->tuning, stream));
+        MC_HIP(launch_layout(w->d_tbl[0], routes, w->d_row_src, w->d_counts, w->stamp[0], d, use_fp8 != 0, w->tuning,
+                             stream));
     }
     if ((phases & MC_EP_PHASE_DATA) && tgrid > 0) {
         PackLaunch pl;
+        pl.row_src = w->d_row_src;
+        pl.counts = w->d_counts;
         if (use_fp8 && w->tuning.scale_mode == 1) {
             if (int rc = ensure_scale_stage(w, (size_t)R * max_tokens * (hidden / 128))) return rc;
             pl.scale_stage = w->d_scale_stage;
@@ -517,6 +540,8 @@ int mc_ep_world_destroy(mc_ep_world_t* w) {
     }
     if (w->d_zero_row) (void)hipFree(w->d_zero_row);
     if (w->d_scale_stage) (void)hipFree(w->d_scale_stage);
+    if (w->d_row_src) (void)hipFree(w->d_row_src);
+    if (w->d_counts) (void)hipFree(w->d_counts);
     if (w->comm_stream) (void)hipStreamDestroy(w->comm_stream);
     delete w;
     return MC_EP_OK;
