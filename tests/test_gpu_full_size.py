@@ -1,0 +1,80 @@
+"""The five named workloads at their full size on the GPU.
+
+Each is compared with the oracle on its valid rows (the oracle finishes a
+whole world in about a second) and through size-independent properties:
+every selection lands exactly once, per-expert counts are the histogram of
+topk_idx, ranges tile [0, count), src_info is ascending inside a range, a
+dispatch -> identity expert -> combine round trip returns x * (sum of unmasked
+weights), and rows beyond recv_count are never written (sampled)."""
+import pytest
+import torch
+
+from mooncake_amd.harness import WorldHarness, valid_rows
+from mooncake_amd.workloads import CONFIG_ORDER, CONFIGS, generate
+from tests import ref_checks as rc
+from tests.gpu_util import announce, compare_dispatch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name", CONFIG_ORDER)
+def test_named_config_full_size(gpu_device, oracle, name):
+    cfg = CONFIGS[name]
+    announce(f"full size {cfg}")
+    data = generate(cfg, seed=0)
+    R, T, E, K, L = cfg.num_ranks, cfg.tokens_per_rank, cfg.num_experts, cfg.num_topk, cfg.num_local_experts
+    RM = R * cfg.max_tokens
+    h = WorldHarness(cfg)
+    h.load(data)
+    h.alloc_dispatch_outputs(poison=False)
+    # sentinel in the row right after each block's expected end, to see that padding is not touched
+    idx = data["topk_idx"]
+    hist = torch.bincount(idx[idx >= 0].flatten(), minlength=E).view(R, L)
+    probe = hist.clamp(max=RM - 1).to(gpu_device)
+    rr = torch.arange(R, device=gpu_device).view(R, 1).expand(R, L)
+    ll = torch.arange(L, device=gpu_device).view(1, L).expand(R, L)
+    h.recv_x[rr, ll, probe] = 0x5C if cfg.use_fp8 else 0x5C5C
+    h.src_info[rr, ll, probe] = -12345
+    h.dispatch()
+    torch.cuda.synchronize()
+
+    # properties
+    cnt = h.recv_count.cpu()
+    assert torch.equal(cnt.to(torch.int64), hist)
+    lr = h.layout_range.cpu()
+    counts, begins = lr & 0xFFFFFFFF, lr >> 32
+    assert torch.equal(counts.sum(dim=2), cnt.to(torch.int64))
+    running = torch.zeros(R, L, dtype=torch.int64)
+    for r in range(R):
+        nz = counts[:, :, r] > 0
+        assert torch.equal(begins[:, :, r][nz], running[nz])
+        running += counts[:, :, r]
+    not_full = (hist < RM).to(gpu_device)
+    assert bool((h.src_info[rr, ll, probe][not_full] == -12345).all())
+    assert bool((h.recv_x[rr, ll, probe][not_full] == (0x5C if cfg.use_fp8 else 0x5C5C)).all())
+
+    # the oracle, on valid rows
+    nt = [T] * R
+    ref = oracle.dispatch(data["x"], idx, nt, cfg.max_tokens, E, cfg.use_fp8, poison=None)
+    compare_dispatch(h, ref, check_poison=False)
+
+    # round trip with the identity expert (bf16) / dequantising expert (fp8)
+    h.alloc_combine_io()
+    h.fill_expert_out_from_recv()
+    h.combine()
+    torch.cuda.synchronize()
+    w = data["topk_weights"].masked_fill(idx == -1, 0).sum(dim=2, keepdim=True)
+    expect = data["x"].float() * w
+    got = h.combined.cpu()
+    if cfg.use_fp8:
+        torch.testing.assert_close(got.float(), expect, rtol=0.15, atol=5e-3 * float(data["x"].float().abs().max()))
+    else:
+        assert rc.calc_diff(expect, got.float()) < 1e-5
+    assert not bool(torch.isnan(got.float()).any())
+    # and bit for bit against the oracle's combine on the same expert outputs (valid rows copied sparsely)
+    eo = torch.empty((R, L, RM, cfg.hidden), dtype=torch.bfloat16)
+    rows = valid_rows(h.expert_out, h.recv_count).cpu()
+    mask = torch.arange(RM).view(1, RM) < cnt.reshape(-1, 1)
+    eo.view(R * L, RM, cfg.hidden)[mask] = rows
+    want = oracle.combine(eo, idx, data["topk_weights"], ref["src_info"], ref["layout_range"], nt, cfg.max_tokens, E)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
