@@ -22,6 +22,15 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 METRIC = "dispatch+combine µs & HBM GB/s (% peak), DSV3 decode 128 tok top-8 fp8"
 
+# HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs of
+# this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what
+# the same counter reads for the library's plain copy kernel over 1 GiB
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Workloads not profiled report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("dsv3_decode", "reduce"): int((230435.4 * 2.0 + 57344.0 * 1.0) * 1024),
+    ("dsv3_decode", "pack"): int((30549.9 * 2.0 + 230322.3 * 1.0) * 1024),
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -34,29 +43,38 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget for the cpu_baseline sample")
     ap.add_argument("--kernel-iters", type=int, default=30, help="timed launches per kernel for the roofline figures")
     ap.add_argument("--opt", action="append", default=[], help="library tuning option, name=value")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="also run the library's plain copy kernel over this many MiB three times (the known-size "
+                         "kernel that profiler FETCH_SIZE / WRITE_SIZE readings are scaled against)")
     return ap.parse_args()
 
 
-def time_kernel(fn, iters, between=None):
-    """Average device time of one launch of `fn`: events on the launch stream
-    around each launch, the stream idle before the start event (so the event
-    pair brackets this launch only); `between` runs untimed before each sample
-    to put the caches in the state the real step leaves them in.  The first
-    sample is dropped."""
+def time_pipeline(h, lib, iters):
+    """Device time of each kernel inside the running dispatch -> combine
+    pipeline: events on the launch stream between the phases of every step, no
+    host synchronisation inside the loop, so each kernel starts on the cache
+    state its predecessor leaves behind (a step moves ~830 MB, far more than L2
+    and the 256 MB memory-side cache hold).  The first two steps are dropped."""
     import torch
-    ms = []
-    for _ in range(iters + 1):
-        if between is not None:
-            between()
-        torch.cuda.synchronize()
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        fn()
-        end.record()
-        end.synchronize()
-        ms.append(start.elapsed_time(end))
-    ms = ms[1:]
-    return sum(ms) / len(ms) * 1e3, min(ms) * 1e3   # microseconds
+    phases = [("layout", h.dispatch, lib.PHASE_LAYOUT), ("pack", h.dispatch, lib.PHASE_DATA),
+              ("scales", h.dispatch, lib.PHASE_FINISH), ("resolve", h.combine, lib.PHASE_LAYOUT),
+              ("reduce", h.combine, lib.PHASE_DATA)]
+    if not h.cfg.use_fp8:
+        phases = [p for p in phases if p[0] != "scales"]
+    marks = []
+    for _ in range(iters + 2):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(len(phases) + 1)]
+        ev[0].record()
+        for i, (_, fn, ph) in enumerate(phases):
+            fn(phases=ph)
+            ev[i + 1].record()
+        marks.append(ev)
+    torch.cuda.synchronize()
+    out = {}
+    for i, (name, _, _) in enumerate(phases):
+        us = [m[i].elapsed_time(m[i + 1]) * 1e3 for m in marks[2:]]
+        out[name] = (sum(us) / len(us), min(us))
+    return out
 
 
 def cpu_baseline(cfg, data, bytes_total, budget_s):
@@ -143,27 +161,14 @@ def main():
     ms_per_step = elapsed / args.steps * 1e3
     step_gbps = (alg["dispatch"] + alg["combine"]) / (elapsed / args.steps) / 1e9
 
-    # per-call and per-kernel device times (events on the launch stream); a
-    # 512 MB write before every sample keeps any launch from starting on a
-    # cache warmed by its own previous run
-    flush = torch.empty(512 * 1024 * 1024 // 4, dtype=torch.int32, device="cuda:0")
-    it = args.kernel_iters
-    d_us, _ = time_kernel(h.dispatch, it, flush.zero_)
-    c_us, _ = time_kernel(h.combine, it, flush.zero_)
-    lay_us, _ = time_kernel(lambda: h.dispatch(phases=_lib.PHASE_LAYOUT), it, flush.zero_)
-    pack_us, pack_min = time_kernel(lambda: h.dispatch(phases=_lib.PHASE_DATA), it, flush.zero_)
-    res_us, _ = time_kernel(lambda: h.combine(phases=_lib.PHASE_LAYOUT), it, flush.zero_)
-    red_us, red_min = time_kernel(lambda: h.combine(phases=_lib.PHASE_DATA), it, flush.zero_)
-    del flush
-
-    kernels = {
-        "pack": {"us": round(pack_us, 2), "min_us": round(pack_min, 2), "bytes": alg["dispatch"],
-                 "GBps": round(alg["dispatch"] / pack_us / 1e3, 1)},
-        "reduce": {"us": round(red_us, 2), "min_us": round(red_min, 2), "bytes": alg["combine"],
-                   "GBps": round(alg["combine"] / red_us / 1e3, 1)},
-        "layout": {"us": round(lay_us, 2)},
-        "resolve": {"us": round(res_us, 2)},
-    }
+    # per-kernel device times, measured live inside the pipeline
+    t = time_pipeline(h, _lib, args.kernel_iters)
+    d_us = sum(t[k][0] for k in ("layout", "pack", "scales") if k in t)
+    c_us = sum(t[k][0] for k in ("resolve", "reduce"))
+    pack_us, red_us = t["pack"][0], t["reduce"][0]
+    kernels = {k: {"us": round(v[0], 2), "min_us": round(v[1], 2)} for k, v in t.items()}
+    kernels["pack"].update(bytes=alg["dispatch"], GBps=round(alg["dispatch"] / pack_us / 1e3, 1))
+    kernels["reduce"].update(bytes=alg["combine"], GBps=round(alg["combine"] / red_us / 1e3, 1))
     # the dominant kernel is the one the step spends most time in
     dom = "reduce" if red_us >= pack_us else "pack"
     achieved = kernels[dom]["GBps"]
@@ -190,8 +195,18 @@ def main():
         "algorithmic_bytes": alg,
         "kernels": kernels,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None},
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((cfg.name, dom)) if not opts else None},
     }
+    if args.copy_calibration > 0:
+        nbytes = args.copy_calibration << 20
+        src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _lib.check(_lib.lib().mc_ep_debug_copy(dst.data_ptr(), src.data_ptr(), nbytes,
+                                                   int(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        out["copy_calibration_bytes"] = nbytes
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, data, alg["dispatch"] + alg["combine"], args.cpu_seconds)
     print(json.dumps(out))

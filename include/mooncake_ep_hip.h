@@ -36,10 +36,12 @@ extern "C" {
 
 /* phases of a whole-world call (the reference's LOW_LATENCY_SEND_PHASE /
  * LOW_LATENCY_RECV_PHASE split, mooncake_ep_configs.cuh:16-17, maps onto the
- * two kernels each call is made of) */
+ * kernels each call is made of; a later phase needs the earlier ones of the
+ * same call to have run) */
 #define MC_EP_PHASE_LAYOUT 1   /* dispatch: routing layout;  combine: handle -> row resolve */
 #define MC_EP_PHASE_DATA 2     /* dispatch: pack;            combine: weighted reduce */
-#define MC_EP_PHASE_ALL 3
+#define MC_EP_PHASE_FINISH 4   /* dispatch: fp8 scales into their column-major layout; combine: nothing */
+#define MC_EP_PHASE_ALL 7
 
 typedef struct mc_ep_world mc_ep_world_t;     /* R logical ranks on one device */
 typedef struct mc_ep_buffer mc_ep_buffer_t;   /* one rank's MooncakeEpBuffer */

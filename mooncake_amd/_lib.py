@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmooncake_ep_hip.so")
 
 OK, ERR_ASSERT, ERR_HIP, ERR_PENDING, ERR_UNSUPPORTED = 0, 1, 2, 3, 4
-PHASE_LAYOUT, PHASE_DATA, PHASE_ALL = 1, 2, 3
+PHASE_LAYOUT, PHASE_DATA, PHASE_FINISH, PHASE_ALL = 1, 2, 4, 7
 
 _lib = None
 

@@ -98,7 +98,8 @@ hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_word
 hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, int32_t* d_row_src, int32_t* d_counts,
                          uint32_t stamp, const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream);
 hipError_t launch_pack(const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp, const PackLaunch& pl,
-                       const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream);
+                       const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
+                       hipStream_t stream);
 hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, const Dims& d,
                           const Tuning& t, hipStream_t stream);
 hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const void* d_zero_row,

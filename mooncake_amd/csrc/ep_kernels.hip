@@ -794,20 +794,23 @@ static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const Dispatch
 }
 
 hipError_t launch_pack(const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp, const PackLaunch& pl,
-                       const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream) {
+                       const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
+                       hipStream_t stream) {
     const bool ntl = t.pack_nt & 1, nts = t.pack_nt & 2;
     float* stage = (use_fp8 && t.scale_mode == 1) ? pl.scale_stage : nullptr;
+    hipError_t err = hipSuccess;
+    if (run_pack) {
 #define MCEP_PACK(KERN)                                                                                \
     (ntl ? (nts ? launch_pack_t(KERN<true, true>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)     \
                 : launch_pack_t(KERN<true, false>, d_tbl, d_routes, stamp, pl, stage, d, t, stream))   \
          : (nts ? launch_pack_t(KERN<false, true>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)    \
                 : launch_pack_t(KERN<false, false>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)))
-    hipError_t err;
     if (!use_fp8) err = MCEP_PACK(pack_bf16_kernel);
     else if (t.pack_variant == 1) err = MCEP_PACK(pack_fp8_split_kernel);
     else err = MCEP_PACK(pack_fp8_kernel);
 #undef MCEP_PACK
-    if (err != hipSuccess || stage == nullptr) return err;
+    }
+    if (err != hipSuccess || stage == nullptr || !run_finish) return err;
     const long long total = (long long)d.E * kTransposeWaves;
     const int wpb = 4;
     LayoutScratch scratch{pl.row_src, pl.counts};

@@ -238,7 +238,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         MC_HIP(launch_layout(w->d_tbl[0], routes, w->d_row_src, w->d_counts, w->stamp[0], d, use_fp8 != 0, w->tuning,
                              stream));
     }
-    if ((phases & MC_EP_PHASE_DATA) && tgrid > 0) {
+    if ((phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
         PackLaunch pl;
         pl.row_src = w->d_row_src;
         pl.counts = w->d_counts;
@@ -256,7 +256,8 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
             pl.x_stride = stride;
             pl.uniform_tokens = num_tokens[0];
         }
-        MC_HIP(launch_pack(w->d_tbl[0], routes, w->stamp[0], pl, d, use_fp8 != 0, w->tuning, stream));
+        MC_HIP(launch_pack(w->d_tbl[0], routes, w->stamp[0], pl, d, use_fp8 != 0, w->tuning,
+                           (phases & MC_EP_PHASE_DATA) != 0, (phases & MC_EP_PHASE_FINISH) != 0, stream));
     }
     return MC_EP_OK;
 }
