@@ -11,6 +11,7 @@ valid (in stream order) once every live rank has made its call.
 """
 from __future__ import annotations
 
+import collections
 from typing import Any, Callable, Optional, Tuple, Union
 
 import torch
@@ -80,6 +81,9 @@ class Buffer:
         self.runtime = ep.Buffer(self.rank, self.group_size, num_ep_buffer_bytes, disable_p2p, world=world)
         # there is no slow path here: the HIP kernels are the only implementation
         self._use_fallback = False
+        # a round may be launched by a later rank's call: keep the tensors of
+        # recent calls alive until then
+        self._keepalive = collections.deque(maxlen=32)
         self.connect()
 
     def connect(self, active_ranks=None) -> None:
@@ -149,9 +153,7 @@ class Buffer:
                   num_experts)
         tensors_to_record = (x, topk_idx, active_ranks, packed_recv_x, packed_recv_x_scales, packed_recv_count,
                              packed_recv_src_info, packed_recv_layout_range)
-        # inputs of a deferred collective must outlive this call: the round
-        # may be launched by a later rank's call
-        self._pending_dispatch_refs = tensors_to_record
+        self._keepalive.append(tensors_to_record)
         return ((packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x, packed_recv_count, handle,
                 EventOverlap(event, tensors_to_record if async_finish else None), hook)
 
@@ -203,7 +205,7 @@ class Buffer:
             topk_weights.size(1), num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy,
             combined_x.data_ptr(), async_finish, return_recv_hook, _native_current_stream_ptr())
         tensors_to_record = (x, topk_idx, topk_weights, active_ranks, src_info, layout_range, combined_x)
-        self._pending_combine_refs = tensors_to_record
+        self._keepalive.append(tensors_to_record)
         return combined_x, EventOverlap(event, tensors_to_record if async_finish else None), hook
 
     def get_next_combine_buffer(self, handle: object):
