@@ -43,21 +43,50 @@ struct TableChunk {
     uint64_t v[kTableChunk];
 };
 
-// What the routing kernels hand to the data kernels: one fully resolved entry
-// per (rank, token, k) selection.  An entry is valid for the launch whose
-// stamp it carries, so entries that no routing thread visits (masked or
-// out-of-range experts, selections absent from a handle) need no clearing pass.
-struct DispatchRoute {      // 32 bytes
-    uint64_t row;           // byte address of the destination payload row
-    uint64_t scale;         // byte address of scales[le][0][row] (fp8)
-    uint32_t stamp;
-    uint32_t pad[3];
+// Routing state a dispatch leaves in world-owned device memory.  The world's
+// selections are cut into units of kUnitSelections consecutive (token, k)
+// entries of one rank (units_per_rank per rank, rank-major).  The count kernel
+// produces, per unit and expert, how many of the unit's selections name the
+// expert and, per selection, its position among those; an exclusive prefix
+// over units turns that into the packed row of every selection:
+//     row(sel) = ubegin[unit(sel)][expert(sel)] + selpos[sel]
+// which is the deterministic order source rank ascending, token ascending.
+constexpr int kUnitSelections = 1024;
+
+struct RoutingScratch {
+    int32_t* ucount;     // [U, E]  selections of unit u that name expert e
+    int32_t* ubegin;     // [U, E]  exclusive prefix of ucount over units
+    int32_t* selpos;     // [R * max_tokens * K]  position inside (unit, expert); -1: no valid expert
+    int32_t* counts;     // [E]     rows per expert (0 for experts of ranks that take no part)
+    int32_t* row_src;    // [E, R * max_tokens]  packed row -> source token slot (rank * max_tokens + token)
+    uint32_t* ticket;    // [1]     blocks of the count kernel that have finished
 };
 
+// One resolved source row of combine's general path (a handle that is not the
+// one the last dispatch produced): valid for the launch whose stamp it carries,
+// so selections that no routing thread visits need no clearing pass.
 struct CombineRoute {       // 16 bytes
     uint64_t src;           // byte address of the expert-output row
     float weight;
     uint32_t stamp;
+};
+
+// Address of a per-rank tensor.  When the ranks' tensors are evenly spaced the
+// address comes from kernel arguments alone (base + rank * stride); otherwise
+// (base == 0) from the rank table, one more dependent load.
+struct RankPtr {
+    uint64_t base = 0;
+    int64_t stride = 0;
+};
+
+struct DispatchSource {
+    RankPtr x, topk_idx;
+    int tokens = -1;        // every rank's token count when they are all equal, else -1 (rank table)
+};
+
+struct CombineSource {
+    RankPtr topk_idx, topk_weights, out;
+    int tokens = -1;
 };
 
 struct Dims {
@@ -67,48 +96,41 @@ struct Dims {
     int H;            // hidden
     int max_tokens;   // num_max_dispatch_tokens_per_rank
     int Tgrid;        // max over ranks of T_r (grid extent in tokens per rank)
+    int units_per_rank() const { return (int)(((long long)max_tokens * K + kUnitSelections - 1) / kUnitSelections); }
+    int units() const { return R * units_per_rank(); }
 };
 
 // Tuning knobs, settable at run time for measurement sweeps.
 struct Tuning {
-    int layout_block = 1024;   // threads per expert block in the layout kernel
-    int layout_rotate = 1;     // start each expert block at its own offset into the selection list
     int pack_variant = 0;      // 0: 32 B/lane loads, 16 B stores; 1: two coalesced 16 B loads, 8 B stores
     int pack_waves = 4;        // waves per block in the pack kernel
     int pack_nt = 1;           // bit 0: streaming (nontemporal) loads, bit 1: streaming stores
-    int pack_uniform = 1;      // take x addresses from kernel arguments when the ranks' x are evenly spaced
+    int uniform = 1;           // take per-rank addresses from kernel arguments when tensors are evenly spaced
     int scale_mode = 1;        // 0: scatter scales from the pack kernel; 1: staged + transposing pass
+    int combine_direct = 1;    // reuse the last dispatch's routing state when combine gets that dispatch's handle
     int combine_chunks = 1;    // 16-byte chunks per lane in the combine kernel
     int combine_waves = 4;     // waves per block in the combine kernel
     int combine_nt = 3;        // bit 0: streaming loads, bit 1: streaming stores
 };
 
-// Per-launch inputs of the pack kernel beyond the rank table.
-struct PackLaunch {
-    uint64_t x_base = 0;        // nonzero: rank r's x is x_base + r * x_stride and every rank has uniform_tokens
-    int64_t x_stride = 0;
-    int uniform_tokens = 0;
-    float* scale_stage = nullptr;   // [R * max_tokens, H / 128] staging rows for fp8 scales
-    int32_t* row_src = nullptr;     // [E, R * max_tokens] packed row -> source token slot, from the layout kernel
-    int32_t* counts = nullptr;      // [E] rows per expert, from the layout kernel
-};
-
 hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_words, hipStream_t stream);
 
-hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, int32_t* d_row_src, int32_t* d_counts,
-                         uint32_t stamp, const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream);
-hipError_t launch_pack(const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp, const PackLaunch& pl,
+hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, const Dims& d,
+                        hipStream_t stream);
+hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, float* scale_stage,
                        const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
                        hipStream_t stream);
 hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, const Dims& d,
                           const Tuning& t, hipStream_t stream);
-hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const void* d_zero_row,
-                         const Dims& d, const Tuning& t, hipStream_t stream);
+// direct: rows come from the last dispatch's routing state (sc); otherwise from d_routes
+hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const RoutingScratch& sc,
+                         bool direct, const CombineSource& src, const void* d_zero_row, const Dims& d, const Tuning& t,
+                         hipStream_t stream);
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 hipError_t launch_fill_u32(void* dst, uint32_t value, size_t words, hipStream_t stream);
 
-// selections (R * max_tokens * K) the layout kernel can hold ballots for in LDS
-constexpr size_t kMaxLayoutLdsBytes = 144 * 1024;
-size_t layout_lds_bytes(const Dims& d);
+// LDS the count kernel needs (per-wave counts and prefixes for every expert)
+constexpr size_t kMaxCountLdsBytes = 144 * 1024;
+size_t count_lds_bytes(const Dims& d);
 
 }  // namespace mcep

@@ -3,10 +3,11 @@
 // payload access is a 16-byte vector load or store that a wave issues over a
 // contiguous span of a row.
 //
-//   layout_kernel   routing layout: per-expert histogram, per-(expert, source
-//                   rank) ranges by prefix sum, source-index map and the
-//                   resolved destination of every (rank, token, k) selection.  Restates the count
-//                   path and the slot assignment of the reference's dispatch
+//   count_kernel    routing layout: per-expert histogram of every 1024-selection
+//                   unit, position of each selection inside it, exclusive
+//                   prefix over units, per-(expert, source rank) ranges and
+//                   per-expert counts.  Restates the count path and the slot
+//                   assignment of the reference's dispatch
 //                   (mooncake-ep/src/mooncake_ep_kernel.cu:274, :319-356,
 //                   :417-437) in a deterministic order: source rank ascending,
 //                   token ascending, as the reference's PyTorch statement has
@@ -99,180 +100,144 @@ __global__ void table_write_kernel(uint64_t* dst, TableChunk chunk, int n) {
 // ---------------------------------------------------------------------------
 // routing layout
 // ---------------------------------------------------------------------------
-// One block per global expert e.  The world's selections form a flat list of
-// 64-entry words, rank-major with a fixed number of words per rank, so that a
-// wave's ballot of "selects e" over one word lists tokens of one source rank in
-// ascending order.  (A token is expected to name an expert at most once; if it
-// names one twice, each occurrence gets its own row, as in the reference
-// kernel, which sends once per k: mooncake_ep_kernel.cu:230,273.)
-//   pass 1  ballots of every word -> LDS.  Each block starts at its own offset
-//           into the list: all E blocks read the same R*T*K indices, and
-//           without the rotation they would all ask the same L2 channel for
-//           the same line at the same time.
-//   scan    exclusive prefix of the per-word popcounts = packed row of the
-//           first hit of each word; rank boundaries give (begin, count).
-//   pass 2  ballot bits -> src_info entries and resolved destination routes.
-struct LayoutScratch {
-    int32_t* row_src;    // [E, R*max]  packed row -> source token slot (rank * max_tokens + token)
-    int32_t* counts;     // [E]         recv_count of every global expert
-};
+__device__ __forceinline__ uint64_t rank_ptr(const uint64_t* __restrict__ tbl, const RankPtr& p, int field, int R,
+                                             int r) {
+    return p.base != 0 ? p.base + (uint64_t)((int64_t)r * p.stride) : tbl[field * R + r];
+}
 
-template <bool FP8>
-__global__ __launch_bounds__(1024) void layout_kernel(const uint64_t* __restrict__ tbl,
-                                                       DispatchRoute* __restrict__ routes, LayoutScratch scratch,
-                                                       uint32_t stamp, int R, int E, int K, int H, int max_tokens,
-                                                       int words_per_rank, int rotate) {
-    extern __shared__ unsigned long long lds[];
-    const int W = R * words_per_rank;
-    unsigned long long* masks = lds;                       // [W]   ballots
-    unsigned long long* rank_idx = lds + W;                // [R]   topk_idx address of each rank
-    int* wbeg = (int*)(rank_idx + R);                      // [W+1] packed row of each word's first hit
-    int* rank_n = wbeg + W + 1;                            // [R]   selections (tokens * K) of each rank
-    int* wave_tot = rank_n + R;                            // [16]
+// One block per unit (1024 consecutive (token, k) selections of one rank), one
+// selection per thread.  Each index is read exactly once.
+//   1. inside a wave, selections naming the same expert are ranked by lane
+//      (one ballot per distinct expert present in the wave);
+//   2. the 16 waves' per-expert counts are prefix-summed in LDS, which gives
+//      every selection its position inside (unit, expert) and the unit its
+//      per-expert histogram;
+// prefix_kernel then turns the units' histograms into packed-row offsets.
+// (A token is expected to name an expert at most once; if it names one twice,
+// each occurrence gets its own row, as in the reference kernel, which sends
+// once per k: mooncake_ep_kernel.cu:230,273.)
+__global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* __restrict__ tbl, RoutingScratch sc,
+                                                                 DispatchSource src, int R, int E, int K,
+                                                                 int max_tokens, int upr) {
+    extern __shared__ unsigned char lds_raw[];
+    constexpr int NW = kUnitSelections / 64;
+    uint16_t* wpre = (uint16_t*)lds_raw;                       // [NW][E] selections of e in earlier waves
+    uint8_t* wcnt = lds_raw + (size_t)NW * E * 2;              // [NW][E] selections of e in the wave
 
-    const int e = blockIdx.x;
-    const int L = E / R, q = e / L, le = e - q * L;
-    // the wave index is wave-uniform: keep it (and all word / rank arithmetic
-    // that follows from it) in scalar registers
-    const int lane = wave_lane(), wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nwaves = blockDim.x >> 6;
+    const int u = blockIdx.x;
+    const int r = u / upr, c = u - r * upr;
+    const int tid = threadIdx.x, lane = wave_lane();
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int T = src.tokens >= 0 ? src.tokens : (int)tbl[DF_NUM_TOKENS * R + r];
+    const int n = T * K;
+    const int sel = c * kUnitSelections + tid;                 // index into the rank's [T, K] list
+
+    int64_t e64 = -1;
+    if (sel < n) e64 = ((const int64_t*)rank_ptr(tbl, src.topk_idx, DF_TOPK_IDX, R, r))[sel];
+    for (int i = tid; i < NW * E / 4; i += kUnitSelections) ((uint32_t*)wcnt)[i] = 0;
+    const bool valid = e64 >= 0 && e64 < (int64_t)E;
+    const int e = valid ? (int)e64 : 0;
+    __syncthreads();
+
+    int rank_in_wave = 0;
+    unsigned long long remaining = __ballot(valid);
+    while (remaining) {
+        const int leader = __builtin_ctzll(remaining);
+        const int e0 = __builtin_amdgcn_readlane(e, leader);
+        const unsigned long long m = __ballot(valid && e == e0);
+        if (valid && e == e0) {
+            rank_in_wave = __popcll(m & ((1ull << lane) - 1ull));
+            if (lane == 63 - __builtin_clzll(m)) wcnt[wave * E + e] = (uint8_t)__popcll(m);
+        }
+        remaining &= ~m;
+    }
+    __syncthreads();
+
+    for (int ee = tid; ee < E; ee += kUnitSelections) {
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            wpre[w * E + ee] = (uint16_t)run;
+            run += wcnt[w * E + ee];
+        }
+        sc.ucount[(int64_t)u * E + ee] = run;
+    }
+    __syncthreads();
+    if (sel < n) sc.selpos[(int64_t)r * max_tokens * K + sel] = valid ? (int)wpre[wave * E + e] + rank_in_wave : -1;
+
+}
+
+// Units' histograms -> exclusive prefixes over units (source rank ascending,
+// then token ascending), recv_count, layout_range and the per-expert counts.
+// One thread per expert; the unit counts are fetched eight at a time.  (A
+// separate launch rather than "the last block of the count kernel": the
+// device-scope release that pattern needs writes back each XCD's whole L2.)
+__global__ __launch_bounds__(64) void prefix_kernel(const uint64_t* __restrict__ tbl, RoutingScratch sc, int R, int E,
+                                                     int max_tokens, int upr, int U) {
+    const int ee = blockIdx.x * blockDim.x + threadIdx.x;
+    if (ee >= E) return;
+    const int L = E / R;
     const int64_t RM = (int64_t)R * max_tokens;
-
-    // a rank that takes no part in this dispatch receives nothing; routes
-    // towards it keep an old stamp and are skipped by the pack kernel
-    const uint64_t recv_x = tbl[DF_RECV_X * R + q];
-    if (recv_x == 0) {
-        if (threadIdx.x == 0) scratch.counts[e] = 0;
-        return;
-    }
-    // the rank table is read once per block, not once per word
-    for (int r = threadIdx.x; r < R; r += blockDim.x) {
-        rank_n[r] = (int)tbl[DF_NUM_TOKENS * R + r] * K;
-        rank_idx[r] = tbl[DF_TOPK_IDX * R + r];
-    }
-    int32_t* recv_count = (int32_t*)tbl[DF_RECV_COUNT * R + q];
-    int32_t* src_info = (int32_t*)tbl[DF_SRC_INFO * R + q] + (int64_t)le * RM;
-    int64_t* layout_range = (int64_t*)tbl[DF_LAYOUT_RANGE * R + q] + (int64_t)le * R;
-    __syncthreads();
-
-    // An item is a run of up to U consecutive words of one rank; a wave takes
-    // IPR items per round and has all their loads in flight before the first ballot.
-    constexpr int U = 8, IPR = 4;
-    const int items_per_rank = (words_per_rank + U - 1) / U;
-    const int items = R * items_per_rank;
-    const int start = rotate ? (int)(((long long)e * items) / E) : 0;
-    for (int it0 = wave * IPR; it0 < items; it0 += nwaves * IPR) {
-        int64_t v[IPR][U];
-        int word0[IPR];
-#pragma unroll
-        for (int a = 0; a < IPR; ++a) {
-            word0[a] = -1;
-            int item = it0 + a;
-            if (item < items) {
-                item += start;
-                if (item >= items) item -= items;
-                const int r = item / items_per_rank, w0 = (item - r * items_per_rank) * U;
-                const int n = rank_n[r];
-                const int64_t* idx = (const int64_t*)rank_idx[r];
-                word0[a] = r * words_per_rank + w0;
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int i = (w0 + u) * 64 + lane;
-                    v[a][u] = (w0 + u < words_per_rank && i < n) ? idx[i] : -1;
-                }
-            } else {
-#pragma unroll
-                for (int u = 0; u < U; ++u) v[a][u] = -1;
-            }
-        }
-#pragma unroll
-        for (int a = 0; a < IPR; ++a) {
-            if (word0[a] < 0) continue;
-            const int w0 = word0[a] % words_per_rank;
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (w0 + u >= words_per_rank) break;
-                const unsigned long long m = __ballot(v[a][u] == (int64_t)e);
-                if (lane == 0) masks[word0[a] + u] = m;
-            }
-        }
-    }
-    __syncthreads();
-
-    // block-wide exclusive scan of the per-word hit counts
-    int carry = 0;
-    for (int base = 0; base < W; base += blockDim.x) {
-        const int gi = base + threadIdx.x;
-        const int c = (gi < W) ? __popcll(masks[gi]) : 0;
-        int incl = c;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const int up = __shfl_up(incl, d);
-            if (lane >= d) incl += up;
-        }
-        if (lane == 63) wave_tot[wave] = incl;
-        __syncthreads();
-        int before = carry;
-        for (int w2 = 0; w2 < wave; ++w2) before += wave_tot[w2];
-        if (gi < W) wbeg[gi] = before + incl - c;
-        int total = 0;
-        for (int w2 = 0; w2 < nwaves; ++w2) total += wave_tot[w2];
-        carry += total;
-        __syncthreads();
-    }
     // A block holds RM rows.  Distinct experts per token can never exceed that;
     // rows past it (possible only with repeated experts) are dropped.
     const int cap = (int)(RM < 0x7fffffff ? RM : 0x7fffffff);
-    if (threadIdx.x == 0) {
-        wbeg[W] = carry;
-        const int kept = carry < cap ? carry : cap;
-        recv_count[le] = kept;
-        scratch.counts[e] = kept;
-    }
-    __syncthreads();
-    for (int r = threadIdx.x; r < R; r += blockDim.x) {
-        int b = wbeg[r * words_per_rank], b2 = wbeg[(r + 1) * words_per_rank];
-        b = b < cap ? b : cap;
-        b2 = b2 < cap ? b2 : cap;
-        const int c = b2 - b;
-        // count in the low half, begin in the high half; an empty pair is 0
-        layout_range[r] = c ? (((int64_t)b << 32) | (int64_t)c) : 0;
-    }
-
-    // Ballot bits -> rows.  32 words per wave step, one per lane; only words
-    // with hits (about one in five for 256 experts) are walked.
-    const uint64_t row_bytes = (uint64_t)H * (FP8 ? 1 : 2);
-    const uint64_t row0 = recv_x + (uint64_t)le * RM * row_bytes;
-    const uint64_t scale0 = FP8 ? tbl[DF_RECV_SCALES * R + q] + (uint64_t)le * (H / 128) * RM * 4 : 0;
-    int32_t* row_src = scratch.row_src + (int64_t)e * RM;
-    for (int base = wave * 32; base < W; base += nwaves * 32) {
-        const int mine = base + (lane & 31);
-        const unsigned long long mword = (mine < W) ? masks[mine] : 0;
-        const int mbeg = (mine < W) ? wbeg[mine] : 0;
-        unsigned int nz = (unsigned int)__ballot(mword != 0);      // lanes 32..63 mirror lanes 0..31
-        while (nz) {
-            const int j = __builtin_ctz(nz);
-            nz &= nz - 1;
-            const unsigned long long m = read_lane_u64(mword, j);
-            const int wb = __builtin_amdgcn_readlane(mbeg, j);
-            if ((m >> lane) & 1ull) {
-                const int pos = wb + __popcll(m & ((1ull << lane) - 1ull));
-                if (pos < cap) {
-                    const int gi = base + j;
-                    const int r = gi / words_per_rank, w = gi - r * words_per_rank;
-                    const int i = w * 64 + lane;
-                    const int t = i / K, k = i - t * K;
-                    src_info[pos] = t;
-                    row_src[pos] = r * max_tokens + t;
-                    DispatchRoute rt;
-                    rt.row = row0 + (uint64_t)pos * row_bytes;
-                    rt.scale = FP8 ? scale0 + (uint64_t)pos * 4 : 0;
-                    rt.stamp = stamp;
-                    rt.pad[0] = rt.pad[1] = rt.pad[2] = 0;
-                    routes[((int64_t)r * max_tokens + t) * K + k] = rt;
-                }
+    const int q = ee / L, le = ee - q * L;
+    const uint64_t recv_x = tbl[DF_RECV_X * R + q];       // 0: the rank takes no part and receives nothing
+    int64_t* layout_range = recv_x ? (int64_t*)tbl[DF_LAYOUT_RANGE * R + q] + (int64_t)le * R : nullptr;
+    int run = 0, rank_begin = 0;
+    for (int u0 = 0; u0 < U; u0 += 8) {
+        int cnt[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) cnt[j] = (u0 + j < U) ? sc.ucount[(int64_t)(u0 + j) * E + ee] : 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int uu = u0 + j;
+            if (uu >= U) break;
+            const int in_rank = uu % upr;
+            if (in_rank == 0) rank_begin = run;
+            sc.ubegin[(int64_t)uu * E + ee] = run;
+            run += cnt[j];
+            if (in_rank == upr - 1 && layout_range != nullptr) {
+                const int b = rank_begin < cap ? rank_begin : cap;
+                const int b2 = run < cap ? run : cap;
+                // count in the low half, begin in the high half; an empty pair is 0
+                layout_range[uu / upr] = (b2 > b) ? (((int64_t)b << 32) | (int64_t)(b2 - b)) : 0;
             }
         }
     }
+    const int kept = run < cap ? run : cap;
+    sc.counts[ee] = recv_x ? kept : 0;
+    if (recv_x) ((int32_t*)tbl[DF_RECV_COUNT * R + q])[le] = kept;
+}
+
+// The packed row of one (token, k) selection, from the routing state.
+struct SelRow {
+    int e;          // global expert
+    int q;          // rank that owns it
+    int64_t grow;   // row inside that rank's [L, R*max] layout: le * R*max + slot
+    int slot;       // row inside the expert's block
+    bool ok;
+};
+
+__device__ __forceinline__ SelRow selection_row(const int64_t* __restrict__ idx_row, const RoutingScratch& sc, int R,
+                                                int E, int K, int max_tokens, int upr, int r, int t, int lane) {
+    SelRow s = {0, 0, 0, 0, false};
+    if (lane < K) {
+        const int i = t * K + lane;
+        const int64_t e64 = idx_row[lane];
+        const int pos = sc.selpos[(int64_t)r * max_tokens * K + i];
+        if (e64 >= 0 && e64 < (int64_t)E && pos >= 0) {
+            const int e = (int)e64, L = E / R;
+            const int u = r * upr + i / kUnitSelections;
+            const int64_t RM = (int64_t)R * max_tokens;
+            s.slot = sc.ubegin[(int64_t)u * E + e] + pos;
+            s.e = e;
+            s.q = e / L;
+            s.grow = (int64_t)(e - s.q * L) * RM + s.slot;
+            s.ok = s.slot < RM;
+        }
+    }
+    return s;
 }
 
 // ---------------------------------------------------------------------------
@@ -286,70 +251,60 @@ struct PackDest {
     uint64_t scale;   // byte address of scales[le][0][slot] (fp8)
 };
 
-// Where a wave finds its token row.  When every rank's x is the same distance
-// from the previous rank's and all ranks hold the same number of tokens, the
-// address comes from kernel arguments alone; otherwise from the rank table
-// (one more dependent scalar load before the row loads can be issued).
-struct PackSource {
-    uint64_t x_base;      // rank 0's x when uniform, else 0
-    int64_t x_stride;     // bytes between consecutive ranks' x
-    int tokens;           // every rank's token count when uniform
-};
-
-__device__ __forceinline__ const char* pack_source_row(const uint64_t* __restrict__ tbl, const PackSource& src, int R,
-                                                       int H, int r, int t, bool* in_range) {
-    if (src.x_base != 0) {
-        *in_range = t < src.tokens;
-        return (const char*)(src.x_base + (uint64_t)((int64_t)r * src.x_stride)) + (int64_t)t * H * 2;
+// Lanes 0..K-1 turn their selection into destination addresses.  The slab-0
+// wave of a token also records the row's source: src_info for the caller and
+// row_src for the scale transposition.
+template <bool FP8>
+__device__ __forceinline__ PackDest pack_destination(const uint64_t* __restrict__ tbl, const RoutingScratch& sc,
+                                                     const int64_t* __restrict__ idx_row, int R, int E, int K,
+                                                     int max_tokens, int H, int upr, int r, int t, int slab,
+                                                     int lane) {
+    PackDest d = {0, 0};
+    const SelRow s = selection_row(idx_row, sc, R, E, K, max_tokens, upr, r, t, lane);
+    if (s.ok) {
+        const uint64_t base = tbl[DF_RECV_X * R + s.q];
+        if (base != 0) {
+            d.row = base + (uint64_t)s.grow * (uint64_t)H * (FP8 ? 1 : 2);
+            if (FP8) {
+                const int64_t RM = (int64_t)R * max_tokens;
+                const int64_t le = s.grow / RM;   // == (grow - slot) / RM
+                d.scale = tbl[DF_RECV_SCALES * R + s.q] + (uint64_t)(le * (H / 128) * RM + s.slot) * 4;
+            }
+            if (slab == 0) {
+                ((int32_t*)tbl[DF_SRC_INFO * R + s.q])[s.grow] = t;
+                sc.row_src[(int64_t)s.e * R * max_tokens + s.slot] = r * max_tokens + t;
+            }
+        }
     }
-    *in_range = t < (int)tbl[DF_NUM_TOKENS * R + r];
-    return (const char*)tbl[DF_X * R + r] + (int64_t)t * H * 2;
-}
-
-struct PackRouteRaw {
-    uint4 a, b;
-};
-
-// issue the route loads (no dependency on anything but the task index) ...
-__device__ __forceinline__ PackRouteRaw pack_route_issue(const DispatchRoute* __restrict__ routes, int K,
-                                                         int max_tokens, int r, int t, int lane) {
-    PackRouteRaw raw = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-    if (lane < K) {
-        const uint4* p = (const uint4*)(routes + ((int64_t)r * max_tokens + t) * K + lane);
-        raw.a = p[0];
-        raw.b = p[1];
-    }
-    return raw;
-}
-
-// ... and consume them after the row loads are in flight.  The empty asm keeps
-// the compiler from fetching the stamp first and the rest behind a branch.
-__device__ __forceinline__ PackDest pack_route_finish(PackRouteRaw raw, uint32_t stamp, int K, int lane) {
-    asm volatile("" : "+v"(raw.a.x), "+v"(raw.a.y), "+v"(raw.a.z), "+v"(raw.a.w), "+v"(raw.b.x));
-    const bool ok = (lane < K) && (raw.b.x == stamp);
-    PackDest d;
-    d.row = ok ? (((uint64_t)raw.a.y << 32) | raw.a.x) : 0;
-    d.scale = ok ? (((uint64_t)raw.a.w << 32) | raw.a.z) : 0;
     return d;
+}
+
+// token row and top-k row of a wave's token; false when the slot is beyond the rank's token count
+__device__ __forceinline__ bool pack_token(const uint64_t* __restrict__ tbl, const DispatchSource& src, int R, int K,
+                                           int H, int r, int t, const char** xrow, const int64_t** idx_row) {
+    const int T = src.tokens >= 0 ? src.tokens : (int)tbl[DF_NUM_TOKENS * R + r];
+    if (t >= T) return false;
+    *xrow = (const char*)rank_ptr(tbl, src.x, DF_X, R, r) + (int64_t)t * H * 2;
+    *idx_row = (const int64_t*)rank_ptr(tbl, src.topk_idx, DF_TOPK_IDX, R, r) + (int64_t)t * K;
+    return true;
 }
 
 // fp8, variant 0: a lane owns 16 consecutive elements (32 B in, 16 B out),
 // a 128-element scale group is 8 lanes.
 template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restrict__ tbl,
-                                                        const DispatchRoute* __restrict__ routes, uint32_t stamp,
-                                                        PackSource src, float* __restrict__ scale_stage, int R,
-                                                        int K, int max_tokens, int H, int slabs, int Tgrid,
+                                                        RoutingScratch sc, DispatchSource src,
+                                                        float* __restrict__ scale_stage, int R, int E, int K,
+                                                        int max_tokens, int H, int upr, int slabs, int Tgrid,
                                                         int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
-    const PackRouteRaw raw = pack_route_issue(routes, K, max_tokens, r, t, lane);
-    bool in_range;
-    const char* xtok = pack_source_row(tbl, src, R, H, r, t, &in_range);
-    if (!in_range) return;
+    const char* xtok;
+    const int64_t* idx_row;
+    if (!pack_token(tbl, src, R, K, H, r, t, &xtok, &idx_row)) return;
 
     const int elem0 = s * 1024 + lane * 16;
     const bool active = elem0 < H;
@@ -359,7 +314,7 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
         a = load16<NTL>(xrow);
         b = load16<NTL>(xrow + 16);
     }
-    const PackDest dst = pack_route_finish(raw, stamp, K, lane);
+    const PackDest dst = pack_destination<true>(tbl, sc, idx_row, R, E, K, max_tokens, H, upr, r, t, s, lane);
 
     float f[16];
     const uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
@@ -406,20 +361,18 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
 // stores are 8 bytes per lane.
 template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __restrict__ tbl,
-                                                              const DispatchRoute* __restrict__ routes,
-                                                              uint32_t stamp, PackSource src,
-                                                              float* __restrict__ scale_stage, int R, int K,
-                                                              int max_tokens, int H, int slabs, int Tgrid,
+                                                              RoutingScratch sc, DispatchSource src,
+                                                              float* __restrict__ scale_stage, int R, int E, int K,
+                                                              int max_tokens, int H, int upr, int slabs, int Tgrid,
                                                               int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
-    const PackRouteRaw raw = pack_route_issue(routes, K, max_tokens, r, t, lane);
-    bool in_range;
-    const char* xbase = pack_source_row(tbl, src, R, H, r, t, &in_range);
-    if (!in_range) return;
+    const char* xbase;
+    const int64_t* idx_row;
+    if (!pack_token(tbl, src, R, K, H, r, t, &xbase, &idx_row)) return;
 
     int elem[2];
     bool active[2];
@@ -431,7 +384,7 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
         v[p] = make_uint4(0, 0, 0, 0);
         if (active[p]) v[p] = load16<NTL>(xbase + (int64_t)elem[p] * 2);
     }
-    const PackDest dst = pack_route_finish(raw, stamp, K, lane);
+    const PackDest dst = pack_destination<true>(tbl, sc, idx_row, R, E, K, max_tokens, H, upr, r, t, s, lane);
 
     uint2 out[2];
     float scale_inv[2];
@@ -482,19 +435,18 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
 // bf16: plain row copy, two unit-stride 16-byte pieces per lane.
 template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restrict__ tbl,
-                                                         const DispatchRoute* __restrict__ routes, uint32_t stamp,
-                                                         PackSource src, float* __restrict__ /*scale_stage*/, int R,
-                                                         int K, int max_tokens, int H, int slabs, int Tgrid,
+                                                         RoutingScratch sc, DispatchSource src,
+                                                         float* __restrict__ /*scale_stage*/, int R, int E, int K,
+                                                         int max_tokens, int H, int upr, int slabs, int Tgrid,
                                                          int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
-    const PackRouteRaw raw = pack_route_issue(routes, K, max_tokens, r, t, lane);
-    bool in_range;
-    const char* xbase = pack_source_row(tbl, src, R, H, r, t, &in_range);
-    if (!in_range) return;
+    const char* xbase;
+    const int64_t* idx_row;
+    if (!pack_token(tbl, src, R, K, H, r, t, &xbase, &idx_row)) return;
 
     int64_t off[2];
     bool active[2];
@@ -507,7 +459,7 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
         v[p] = make_uint4(0, 0, 0, 0);
         if (active[p]) v[p] = load16<NTL>(xbase + off[p]);
     }
-    const PackDest dst = pack_route_finish(raw, stamp, K, lane);
+    const PackDest dst = pack_destination<false>(tbl, sc, idx_row, R, E, K, max_tokens, H, upr, r, t, s, lane);
 
     for (int k = 0; k < K; ++k) {
         const uint64_t row = read_lane_u64(dst.row, k);
@@ -520,14 +472,14 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
 
 // Staged scales -> column-major output.  kTransposeWaves waves per expert,
 // each taking 64 packed rows at a time: a lane learns its row's source token
-// slot from the layout kernel's row_src, reads that token's H/128 scales as
+// slot from row_src (left by the pack kernel), reads that token's H/128 scales as
 // contiguous 16-byte pieces - a batch of them in flight at once - and stores
 // them so that the wave writes 64 consecutive floats per scale group.
 constexpr int kTransposeWaves = 8;
 
 __global__ __launch_bounds__(256) void scale_transpose_kernel(const uint64_t* __restrict__ tbl,
                                                                const float* __restrict__ scale_stage,
-                                                               LayoutScratch scratch, int R, int E, int G,
+                                                               RoutingScratch scratch, int R, int E, int G,
                                                                int max_tokens, int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
@@ -641,32 +593,56 @@ __global__ __launch_bounds__(256) void resolve_kernel(const uint64_t* __restrict
     }
 }
 
-// One wave per (token, slab of CH * 512 elements).  Lanes 0..K-1 fetch the K
-// routes (a masked, inactive or unknown selection reads a zero row with
+// One wave per (token, slab of CH * 512 elements).  Lanes 0..K-1 find the K
+// source rows (a masked, inactive or unknown selection reads a zero row with
 // weight 0, which leaves the fp32 accumulator unchanged), then every lane
 // issues all KMAX * CH 16-byte loads before the first multiply-add.
-template <int KMAX, int CH, bool NTL, bool NTS>
+//   DIRECT   the handle is the one the last dispatch produced: rows come from
+//            that dispatch's routing state, no resolve kernel has run;
+//   !DIRECT  rows come from the routes the resolve kernel left.
+template <int KMAX, int CH, bool NTL, bool NTS, bool DIRECT>
 __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict__ tbl,
                                                       const CombineRoute* __restrict__ routes, uint32_t stamp,
-                                                      const void* __restrict__ zero_row, int R, int K,
-                                                      int max_tokens, int H, int slabs, int Tgrid, int total_tasks) {
+                                                      RoutingScratch sc, CombineSource cs,
+                                                      const void* __restrict__ zero_row, int R, int E, int K,
+                                                      int max_tokens, int H, int upr, int slabs, int Tgrid,
+                                                      int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
-    // A token slot beyond the rank's count has only stale routes (zero rows);
-    // it is computed like any other and dropped at the store, so that no wave
-    // waits for the rank's token count before it can issue its loads.
-    const int T = (int)tbl[CF_NUM_TOKENS * R + r];
-    char* orow = (char*)tbl[CF_OUT * R + r] + (int64_t)t * H * 2;
+    const int T = cs.tokens >= 0 ? cs.tokens : (int)tbl[CF_NUM_TOKENS * R + r];
+    char* orow = (char*)rank_ptr(tbl, cs.out, CF_OUT, R, r) + (int64_t)t * H * 2;
 
-    uint4 rt = make_uint4(0, 0, 0, 0);
-    if (lane < K) rt = *(const uint4*)(routes + ((int64_t)r * max_tokens + t) * K + lane);
-    asm volatile("" : "+v"(rt.x), "+v"(rt.y), "+v"(rt.z), "+v"(rt.w));   // one 16-byte load, no branch on the stamp
-    const bool ok = (lane < K) && (rt.w == stamp);
-    const uint64_t src = ok ? (((uint64_t)rt.y << 32) | rt.x) : (uint64_t)zero_row;
-    const float w = ok ? __uint_as_float(rt.z) : 0.0f;
+    uint64_t src = (uint64_t)zero_row;
+    float w = 0.0f;
+    if (DIRECT) {
+        // the caller's top-k rows exist only for t < T
+        if (t >= T) return;
+        const int64_t* idx_row = (const int64_t*)rank_ptr(tbl, cs.topk_idx, CF_TOPK_IDX, R, r) + (int64_t)t * K;
+        const float* w_row = (const float*)rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (int64_t)t * K;
+        const float wl = (lane < K) ? w_row[lane] : 0.0f;
+        const SelRow sr = selection_row(idx_row, sc, R, E, K, max_tokens, upr, r, t, lane);
+        if (sr.ok) {
+            const uint64_t base = tbl[CF_X * R + sr.q];
+            const int live = ((const int32_t*)tbl[CF_ACTIVE * R + r])[sr.q];   // skip experts on inactive ranks
+            if (base != 0 && live != 0) {
+                src = base + (uint64_t)sr.grow * (uint64_t)H * 2;
+                w = wl;
+            }
+        }
+    } else {
+        // A token slot beyond the rank's count has only stale routes (zero
+        // rows); it is computed like any other and dropped at the store, so
+        // that no wave waits for the rank's token count before its loads.
+        uint4 rt = make_uint4(0, 0, 0, 0);
+        if (lane < K) rt = *(const uint4*)(routes + ((int64_t)r * max_tokens + t) * K + lane);
+        asm volatile("" : "+v"(rt.x), "+v"(rt.y), "+v"(rt.z), "+v"(rt.w));   // one 16-byte load, no branch on the stamp
+        const bool ok = (lane < K) && (rt.w == stamp);
+        src = ok ? (((uint64_t)rt.y << 32) | rt.x) : (uint64_t)zero_row;
+        w = ok ? __uint_as_float(rt.z) : 0.0f;
+    }
 
     int64_t off[CH];
     bool active[CH];
@@ -746,76 +722,66 @@ hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_word
     return hipSuccess;
 }
 
-size_t layout_lds_bytes(const Dims& d) {
-    const size_t words_per_rank = ((size_t)d.max_tokens * d.K + 63) / 64;
-    const size_t W = (size_t)d.R * words_per_rank;
-    return W * 8 + (size_t)d.R * 8 + (W + 1) * 4 + (size_t)d.R * 4 + 16 * 4 + 16;
+size_t count_lds_bytes(const Dims& d) {
+    return (size_t)(kUnitSelections / 64) * d.E * 3 + 64;
 }
 
-hipError_t launch_layout(const uint64_t* d_tbl, DispatchRoute* d_routes, int32_t* d_row_src, int32_t* d_counts,
-                         uint32_t stamp, const Dims& d, bool use_fp8, const Tuning& t, hipStream_t stream) {
-    const size_t lds = layout_lds_bytes(d);
-    if (lds > kMaxLayoutLdsBytes) return hipErrorInvalidValue;
-    const int words_per_rank = (int)(((size_t)d.max_tokens * d.K + 63) / 64);
-    int block = t.layout_block;
-    if (block < 64) block = 64;
-    if (block > 1024) block = 1024;
-    block &= ~63;
-    auto kern = use_fp8 ? layout_kernel<true> : layout_kernel<false>;
+hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, const Dims& d,
+                        hipStream_t stream) {
+    const size_t lds = count_lds_bytes(d);
+    if (lds > kMaxCountLdsBytes) return hipErrorInvalidValue;
     if (lds > 48 * 1024) {
-        hipError_t err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t err =
+            hipFuncSetAttribute((const void*)count_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
     }
-    LayoutScratch scratch{d_row_src, d_counts};
-    hipLaunchKernelGGL(kern, dim3(d.E), dim3(block), lds, stream, d_tbl, d_routes, scratch, stamp, d.R, d.E, d.K,
-                       d.H, d.max_tokens, words_per_rank, t.layout_rotate);
+    hipLaunchKernelGGL(count_kernel, dim3(d.units()), dim3(kUnitSelections), lds, stream, d_tbl, sc, src, d.R, d.E,
+                       d.K, d.max_tokens, d.units_per_rank());
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    hipLaunchKernelGGL(prefix_kernel, dim3((d.E + 63) / 64), dim3(64), 0, stream, d_tbl, sc, d.R, d.E, d.max_tokens,
+                       d.units_per_rank(), d.units());
     return hipGetLastError();
 }
 
 static int clamp_waves(int w) { return w < 1 ? 1 : (w > 8 ? 8 : w); }
 
 template <typename Kern>
-static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp,
-                                const PackLaunch& pl, float* stage, const Dims& d, const Tuning& t,
-                                hipStream_t stream) {
+static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src,
+                                float* stage, const Dims& d, const Tuning& t, hipStream_t stream) {
     const int slabs = (d.H + 1023) / 1024;
     const long long total = (long long)d.R * d.Tgrid * slabs;
     if (total <= 0) return hipSuccess;
     if (total > 0x7fffffffll) return hipErrorInvalidValue;
     const int wpb = clamp_waves(t.pack_waves);
     const int blocks = (int)((total + wpb - 1) / wpb);
-    PackSource src;
-    src.x_base = pl.x_base;
-    src.x_stride = pl.x_stride;
-    src.tokens = pl.uniform_tokens;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_routes, stamp, src, stage, d.R, d.K,
-                       d.max_tokens, d.H, slabs, d.Tgrid, (int)total);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, sc, src, stage, d.R, d.E, d.K,
+                       d.max_tokens, d.H, d.units_per_rank(), slabs, d.Tgrid, (int)total);
     return hipGetLastError();
 }
 
-hipError_t launch_pack(const uint64_t* d_tbl, const DispatchRoute* d_routes, uint32_t stamp, const PackLaunch& pl,
+hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, float* scale_stage,
                        const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
                        hipStream_t stream) {
     const bool ntl = t.pack_nt & 1, nts = t.pack_nt & 2;
-    float* stage = (use_fp8 && t.scale_mode == 1) ? pl.scale_stage : nullptr;
+    float* stage = (use_fp8 && t.scale_mode == 1) ? scale_stage : nullptr;
     hipError_t err = hipSuccess;
     if (run_pack) {
-#define MCEP_PACK(KERN)                                                                                \
-    (ntl ? (nts ? launch_pack_t(KERN<true, true>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)     \
-                : launch_pack_t(KERN<true, false>, d_tbl, d_routes, stamp, pl, stage, d, t, stream))   \
-         : (nts ? launch_pack_t(KERN<false, true>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)    \
-                : launch_pack_t(KERN<false, false>, d_tbl, d_routes, stamp, pl, stage, d, t, stream)))
-    if (!use_fp8) err = MCEP_PACK(pack_bf16_kernel);
-    else if (t.pack_variant == 1) err = MCEP_PACK(pack_fp8_split_kernel);
-    else err = MCEP_PACK(pack_fp8_kernel);
+#define MCEP_PACK(KERN)                                                                          \
+    (ntl ? (nts ? launch_pack_t(KERN<true, true>, d_tbl, sc, src, stage, d, t, stream)           \
+                : launch_pack_t(KERN<true, false>, d_tbl, sc, src, stage, d, t, stream))         \
+         : (nts ? launch_pack_t(KERN<false, true>, d_tbl, sc, src, stage, d, t, stream)          \
+                : launch_pack_t(KERN<false, false>, d_tbl, sc, src, stage, d, t, stream)))
+        if (!use_fp8) err = MCEP_PACK(pack_bf16_kernel);
+        else if (t.pack_variant == 1) err = MCEP_PACK(pack_fp8_split_kernel);
+        else err = MCEP_PACK(pack_fp8_kernel);
 #undef MCEP_PACK
     }
     if (err != hipSuccess || stage == nullptr || !run_finish) return err;
     const long long total = (long long)d.E * kTransposeWaves;
     const int wpb = 4;
-    LayoutScratch scratch{pl.row_src, pl.counts};
     hipLaunchKernelGGL(scale_transpose_kernel, dim3((unsigned)((total + wpb - 1) / wpb)), dim3(wpb * 64), 0, stream,
-                       d_tbl, stage, scratch, d.R, d.E, d.H / 128, d.max_tokens, (int)total);
+                       d_tbl, stage, sc, d.R, d.E, d.H / 128, d.max_tokens, (int)total);
     return hipGetLastError();
 }
 
@@ -831,9 +797,19 @@ hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_
     return hipGetLastError();
 }
 
-template <int KMAX, int CH>
-static hipError_t launch_reduce_t(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp,
-                                  const void* d_zero_row, const Dims& d, const Tuning& t, hipStream_t stream) {
+namespace {
+struct ReduceLaunch {
+    const uint64_t* d_tbl;
+    const CombineRoute* d_routes;
+    uint32_t stamp;
+    RoutingScratch sc;
+    CombineSource src;
+    const void* d_zero_row;
+};
+}  // namespace
+
+template <int KMAX, int CH, bool DIRECT>
+static hipError_t launch_reduce_t(const ReduceLaunch& rl, const Dims& d, const Tuning& t, hipStream_t stream) {
     const int slabs = (d.H + CH * 512 - 1) / (CH * 512);
     const long long total = (long long)d.R * d.Tgrid * slabs;
     if (total <= 0) return hipSuccess;
@@ -841,9 +817,10 @@ static hipError_t launch_reduce_t(const uint64_t* d_tbl, const CombineRoute* d_r
     const int wpb = clamp_waves(t.combine_waves);
     const int blocks = (int)((total + wpb - 1) / wpb);
     const bool ntl = t.combine_nt & 1, nts = t.combine_nt & 2;
-#define MCEP_REDUCE(A, B)                                                                                       \
-    hipLaunchKernelGGL((reduce_kernel<KMAX, CH, A, B>), dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_routes, \
-                       stamp, d_zero_row, d.R, d.K, d.max_tokens, d.H, slabs, d.Tgrid, (int)total)
+#define MCEP_REDUCE(A, B)                                                                                        \
+    hipLaunchKernelGGL((reduce_kernel<KMAX, CH, A, B, DIRECT>), dim3(blocks), dim3(wpb * 64), 0, stream, rl.d_tbl, \
+                       rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d.R, d.E, d.K, d.max_tokens, d.H,    \
+                       d.units_per_rank(), slabs, d.Tgrid, (int)total)
     if (ntl && nts) MCEP_REDUCE(true, true);
     else if (ntl) MCEP_REDUCE(true, false);
     else if (nts) MCEP_REDUCE(false, true);
@@ -852,18 +829,24 @@ static hipError_t launch_reduce_t(const uint64_t* d_tbl, const CombineRoute* d_r
     return hipGetLastError();
 }
 
-hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const void* d_zero_row,
-                         const Dims& d, const Tuning& t, hipStream_t stream) {
+hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const RoutingScratch& sc,
+                         bool direct, const CombineSource& src, const void* d_zero_row, const Dims& d, const Tuning& t,
+                         hipStream_t stream) {
+    const ReduceLaunch rl{d_tbl, d_routes, stamp, sc, src, d_zero_row};
     const int ch = t.combine_chunks >= 2 ? 2 : 1;
-#define MCEP_K(KMAX)                                                                                    \
-    return ch == 2 ? launch_reduce_t<KMAX, 2>(d_tbl, d_routes, stamp, d_zero_row, d, t, stream)         \
-                   : launch_reduce_t<KMAX, 1>(d_tbl, d_routes, stamp, d_zero_row, d, t, stream)
-    if (d.K <= 1) { MCEP_K(1); }
-    if (d.K <= 2) { MCEP_K(2); }
-    if (d.K <= 4) { MCEP_K(4); }
-    if (d.K <= 6) { MCEP_K(6); }
-    if (d.K <= 8) { MCEP_K(8); }
-    if (d.K <= 12) { MCEP_K(12); }
+#define MCEP_K(KMAX)                                                                                   \
+    do {                                                                                               \
+        if (direct) return ch == 2 ? launch_reduce_t<KMAX, 2, true>(rl, d, t, stream)                  \
+                                   : launch_reduce_t<KMAX, 1, true>(rl, d, t, stream);                 \
+        return ch == 2 ? launch_reduce_t<KMAX, 2, false>(rl, d, t, stream)                             \
+                       : launch_reduce_t<KMAX, 1, false>(rl, d, t, stream);                            \
+    } while (0)
+    if (d.K <= 1) MCEP_K(1);
+    if (d.K <= 2) MCEP_K(2);
+    if (d.K <= 4) MCEP_K(4);
+    if (d.K <= 6) MCEP_K(6);
+    if (d.K <= 8) MCEP_K(8);
+    if (d.K <= 12) MCEP_K(12);
     MCEP_K(16);
 #undef MCEP_K
 }

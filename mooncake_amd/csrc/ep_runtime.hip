@@ -83,13 +83,30 @@ struct mc_ep_world {
     hipStream_t comm_stream = nullptr;
     uint64_t* d_tbl[2] = {nullptr, nullptr};     // dispatch, combine pointer tables
     std::vector<uint64_t> tbl_cache[2];           // what the device tables hold
-    void* d_routes[2] = {nullptr, nullptr};      // per-selection routes: DispatchRoute[], CombineRoute[]
-    size_t route_cap[2] = {0, 0};                 // capacity in selections
-    uint32_t stamp[2] = {0, 0};                   // launch counter the routes are stamped with
-    int32_t* d_row_src = nullptr;                 // [E, R*max] packed row -> source token slot
+    // routing state of the last dispatch (see RoutingScratch)
+    int32_t* d_ucount = nullptr;
+    size_t ucount_cap = 0;
+    int32_t* d_ubegin = nullptr;
+    size_t ubegin_cap = 0;
+    int32_t* d_selpos = nullptr;
+    size_t selpos_cap = 0;
+    int32_t* d_row_src = nullptr;
     size_t row_src_cap = 0;
-    int32_t* d_counts = nullptr;                  // [E] rows per expert of the last layout
+    int32_t* d_counts = nullptr;
     size_t counts_cap = 0;
+    uint32_t* d_ticket = nullptr;
+    size_t ticket_cap = 0;
+    // what the last dispatch was called with, so that a combine given that
+    // dispatch's handle can reuse its routing state instead of re-deriving rows
+    struct LastDispatch {
+        bool valid = false;
+        int hidden = 0, num_topk = 0, max_tokens = 0, num_experts = 0;
+        std::vector<uint64_t> topk_idx, recv_x, src_info, layout_range;
+        std::vector<int32_t> num_tokens;
+    } last;
+    CombineRoute* d_routes = nullptr;             // combine's general path: one route per selection
+    size_t route_cap = 0;                         // capacity in selections
+    uint32_t stamp = 0;                           // launch counter the routes are stamped with
     float* d_scale_stage = nullptr;               // fp8 scales of each token before transposition
     size_t scale_stage_cap = 0;                   // capacity in floats
     void* d_zero_row = nullptr;
@@ -132,20 +149,19 @@ struct DeviceGuard {
     }
 };
 
-int ensure_routes(mc_ep_world* w, int which, size_t selections) {
-    if (selections <= w->route_cap[which]) return MC_EP_OK;
+int ensure_routes(mc_ep_world* w, size_t selections) {
+    if (selections <= w->route_cap) return MC_EP_OK;
     // grows only; the old table may still be read by queued kernels
     MC_HIP(hipDeviceSynchronize());
-    if (w->d_routes[which]) MC_HIP(hipFree(w->d_routes[which]));
-    w->d_routes[which] = nullptr;
-    w->route_cap[which] = 0;
+    if (w->d_routes) MC_HIP(hipFree(w->d_routes));
+    w->d_routes = nullptr;
+    w->route_cap = 0;
     const size_t cap = selections + selections / 2 + 1024;
-    const size_t bytes = cap * (which == 0 ? sizeof(DispatchRoute) : sizeof(CombineRoute));
-    MC_HIP(hipMalloc(&w->d_routes[which], bytes));
+    MC_HIP(hipMalloc((void**)&w->d_routes, cap * sizeof(CombineRoute)));
     // stamps start at 1, so a zeroed table holds no valid route
-    MC_HIP(hipMemset(w->d_routes[which], 0, bytes));
-    w->stamp[which] = 0;
-    w->route_cap[which] = cap;
+    MC_HIP(hipMemset(w->d_routes, 0, cap * sizeof(CombineRoute)));
+    w->stamp = 0;
+    w->route_cap = cap;
     return MC_EP_OK;
 }
 
@@ -193,6 +209,30 @@ int check_dims(const mc_ep_world* w, int hidden, int num_topk, int max_tokens, i
     return MC_EP_OK;
 }
 
+// Evenly spaced per-rank tensors (every rank present) can be addressed from
+// kernel arguments; otherwise base stays 0 and kernels use the rank table.
+RankPtr uniform_ptr(const uint64_t* p, int R, bool enabled) {
+    RankPtr u;
+    if (!enabled || p[0] == 0) return u;
+    const int64_t stride = R > 1 ? (int64_t)(p[1] - p[0]) : 0;
+    for (int r = 0; r < R; ++r)
+        if (p[r] == 0 || p[r] != p[0] + (uint64_t)(stride * r)) return u;
+    u.base = p[0];
+    u.stride = stride;
+    return u;
+}
+
+int uniform_tokens(const int32_t* n, int R, bool enabled) {
+    if (!enabled) return -1;
+    for (int r = 1; r < R; ++r)
+        if (n[r] != n[0]) return -1;
+    return n[0];
+}
+
+RoutingScratch routing_scratch(const mc_ep_world* w) {
+    return RoutingScratch{w->d_ucount, w->d_ubegin, w->d_selpos, w->d_counts, w->d_row_src, w->d_ticket};
+}
+
 int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_idx, const int32_t* num_tokens,
                         int hidden, int num_topk, int max_tokens, int num_experts, int use_fp8,
                         const uint64_t* recv_x, const uint64_t* recv_scales, const uint64_t* recv_count,
@@ -226,37 +266,41 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     }
     DeviceGuard guard(w->device);
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
-    // the layout kernel keeps one ballot per 64 selections of the world in LDS
-    MC_ASSERT(layout_lds_bytes(d) <= kMaxLayoutLdsBytes);
-    if (int rc = ensure_routes(w, 0, (size_t)R * max_tokens * num_topk)) return rc;
+    // the count kernel keeps per-wave counts and prefixes of every expert in LDS
+    MC_ASSERT(count_lds_bytes(d) <= kMaxCountLdsBytes);
+    const size_t UE = (size_t)d.units() * num_experts;
+    if (int rc = ensure_scratch(&w->d_ucount, &w->ucount_cap, UE)) return rc;
+    if (int rc = ensure_scratch(&w->d_ubegin, &w->ubegin_cap, UE)) return rc;
+    if (int rc = ensure_scratch(&w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
     if (int rc = ensure_scratch(&w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
     if (int rc = ensure_scratch(&w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
+    if (int rc = ensure_scratch(&w->d_ticket, &w->ticket_cap, (size_t)1)) return rc;
     if (int rc = upload_table(w, 0, tbl, stream)) return rc;
-    auto* routes = (DispatchRoute*)w->d_routes[0];
+
+    const bool uni = w->tuning.uniform != 0;
+    DispatchSource src;
+    src.x = uniform_ptr(x, R, uni);
+    src.topk_idx = uniform_ptr(topk_idx, R, uni);
+    src.tokens = uniform_tokens(num_tokens, R, uni);
+    const RoutingScratch sc = routing_scratch(w);
     if (phases & MC_EP_PHASE_LAYOUT) {
-        w->stamp[0] += 1;
-        MC_HIP(launch_layout(w->d_tbl[0], routes, w->d_row_src, w->d_counts, w->stamp[0], d, use_fp8 != 0, w->tuning,
-                             stream));
+        MC_HIP(launch_count(w->d_tbl[0], sc, src, d, stream));
+        auto& ld = w->last;
+        ld.valid = true;
+        ld.hidden = hidden; ld.num_topk = num_topk; ld.max_tokens = max_tokens; ld.num_experts = num_experts;
+        ld.topk_idx.assign(topk_idx, topk_idx + R);
+        ld.recv_x.assign(recv_x, recv_x + R);
+        ld.src_info.assign(src_info, src_info + R);
+        ld.layout_range.assign(layout_range, layout_range + R);
+        ld.num_tokens.assign(num_tokens, num_tokens + R);
     }
     if ((phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
-        PackLaunch pl;
-        pl.row_src = w->d_row_src;
-        pl.counts = w->d_counts;
+        float* stage = nullptr;
         if (use_fp8 && w->tuning.scale_mode == 1) {
             if (int rc = ensure_scale_stage(w, (size_t)R * max_tokens * (hidden / 128))) return rc;
-            pl.scale_stage = w->d_scale_stage;
+            stage = w->d_scale_stage;
         }
-        // evenly spaced x tensors with one token count: addresses from kernel arguments
-        bool uniform = w->tuning.pack_uniform != 0 && x[0] != 0;
-        const int64_t stride = R > 1 ? (int64_t)(x[1] - x[0]) : 0;
-        for (int r = 0; r < R && uniform; ++r)
-            uniform = num_tokens[r] == num_tokens[0] && x[r] == x[0] + (uint64_t)(stride * r);
-        if (uniform) {
-            pl.x_base = x[0];
-            pl.x_stride = stride;
-            pl.uniform_tokens = num_tokens[0];
-        }
-        MC_HIP(launch_pack(w->d_tbl[0], routes, w->stamp[0], pl, d, use_fp8 != 0, w->tuning,
+        MC_HIP(launch_pack(w->d_tbl[0], sc, src, stage, d, use_fp8 != 0, w->tuning,
                            (phases & MC_EP_PHASE_DATA) != 0, (phases & MC_EP_PHASE_FINISH) != 0, stream));
     }
     return MC_EP_OK;
@@ -292,16 +336,39 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     }
     if (tgrid == 0) return MC_EP_OK;
     DeviceGuard guard(w->device);
-    if (int rc = ensure_routes(w, 1, (size_t)R * max_tokens * num_topk)) return rc;
     if (int rc = upload_table(w, 1, tbl, stream)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
-    auto* routes = (CombineRoute*)w->d_routes[1];
-    if (phases & MC_EP_PHASE_LAYOUT) {
-        w->stamp[1] += 1;
-        MC_HIP(launch_resolve(w->d_tbl[1], routes, w->stamp[1], d, w->tuning, stream));
+
+    // Is this the handle (and the routing input) of the last dispatch?  Then the
+    // packed row of every selection is already known on the device.  Like the
+    // reference, this relies on topk_idx being unchanged between a dispatch and
+    // the combine of its handle (mooncake_ep_kernel.cu:734 finds a token's rows
+    // by its dispatch-time expert indices).
+    const auto& ld = w->last;
+    bool direct = w->tuning.combine_direct != 0 && ld.valid && ld.hidden == hidden && ld.num_topk == num_topk &&
+                  ld.max_tokens == max_tokens && ld.num_experts == num_experts;
+    for (int r = 0; r < R && direct; ++r) {
+        if (num_tokens[r] > 0) direct = topk_idx[r] == ld.topk_idx[r] && num_tokens[r] == ld.num_tokens[r];
+        if (direct && x[r] != 0)
+            direct = ld.recv_x[r] != 0 && src_info[r] == ld.src_info[r] && layout_range[r] == ld.layout_range[r];
+    }
+
+    const bool uni = w->tuning.uniform != 0;
+    CombineSource src;
+    src.topk_idx = uniform_ptr(topk_idx, R, uni);
+    src.topk_weights = uniform_ptr(topk_weights, R, uni);
+    src.out = uniform_ptr(out, R, uni);
+    src.tokens = uniform_tokens(num_tokens, R, uni);
+    if (!direct) {
+        if (int rc = ensure_routes(w, (size_t)R * max_tokens * num_topk)) return rc;
+        if (phases & MC_EP_PHASE_LAYOUT) {
+            w->stamp += 1;
+            MC_HIP(launch_resolve(w->d_tbl[1], w->d_routes, w->stamp, d, w->tuning, stream));
+        }
     }
     if (phases & MC_EP_PHASE_DATA)
-        MC_HIP(launch_reduce(w->d_tbl[1], routes, w->stamp[1], w->d_zero_row, d, w->tuning, stream));
+        MC_HIP(launch_reduce(w->d_tbl[1], w->d_routes, w->stamp, routing_scratch(w), direct, src, w->d_zero_row, d,
+                             w->tuning, stream));
     return MC_EP_OK;
 }
 
@@ -535,10 +602,13 @@ int mc_ep_world_destroy(mc_ep_world_t* w) {
     if (!w) return MC_EP_OK;
     DeviceGuard guard(w->device);
     (void)hipDeviceSynchronize();
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 2; ++i)
         if (w->d_tbl[i]) (void)hipFree(w->d_tbl[i]);
-        if (w->d_routes[i]) (void)hipFree(w->d_routes[i]);
-    }
+    if (w->d_routes) (void)hipFree(w->d_routes);
+    if (w->d_ucount) (void)hipFree(w->d_ucount);
+    if (w->d_ubegin) (void)hipFree(w->d_ubegin);
+    if (w->d_selpos) (void)hipFree(w->d_selpos);
+    if (w->d_ticket) (void)hipFree(w->d_ticket);
     if (w->d_zero_row) (void)hipFree(w->d_zero_row);
     if (w->d_scale_stage) (void)hipFree(w->d_scale_stage);
     if (w->d_row_src) (void)hipFree(w->d_row_src);
@@ -559,15 +629,14 @@ int mc_ep_world_set_rank_silent(mc_ep_world_t* w, int rank, int silent) {
 }
 
 static int* option_slot(Tuning& t, const char* name) {
-    if (!strcmp(name, "layout_block")) return &t.layout_block;
-    if (!strcmp(name, "layout_rotate")) return &t.layout_rotate;
     if (!strcmp(name, "pack_variant")) return &t.pack_variant;
     if (!strcmp(name, "pack_waves")) return &t.pack_waves;
+    if (!strcmp(name, "pack_nt")) return &t.pack_nt;
+    if (!strcmp(name, "uniform")) return &t.uniform;
     if (!strcmp(name, "scale_mode")) return &t.scale_mode;
+    if (!strcmp(name, "combine_direct")) return &t.combine_direct;
     if (!strcmp(name, "combine_chunks")) return &t.combine_chunks;
     if (!strcmp(name, "combine_waves")) return &t.combine_waves;
-    if (!strcmp(name, "pack_nt")) return &t.pack_nt;
-    if (!strcmp(name, "pack_uniform")) return &t.pack_uniform;
     if (!strcmp(name, "combine_nt")) return &t.combine_nt;
     return nullptr;
 }

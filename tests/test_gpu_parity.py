@@ -52,13 +52,12 @@ def test_fp8_pack_variants_match_oracle(gpu_device, oracle, variant, nt, scale_m
     announce(f"pack variant={variant} nt={nt} scale_mode={scale_mode} uniform={uniform}")
     data = generate(cfg, seed=1)
     h = run_dispatch(cfg, data, poison=True, options={"pack_variant": variant, "pack_nt": nt,
-                                                      "scale_mode": scale_mode, "pack_uniform": uniform})
+                                                      "scale_mode": scale_mode, "uniform": uniform})
     ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, True)
     compare_dispatch(h, ref, check_poison=True)
 
 
-@pytest.mark.parametrize("opts", [{"layout_rotate": 0}, {"layout_block": 256}, {"layout_block": 64},
-                                  {"pack_waves": 1}, {"pack_waves": 8}, {"pack_nt": 1}, {"pack_nt": 2}],
+@pytest.mark.parametrize("opts", [{"uniform": 0}, {"pack_waves": 1}, {"pack_waves": 8}, {"pack_nt": 1}, {"pack_nt": 2}],
                          ids=lambda o: "-".join(f"{k}{v}" for k, v in o.items()))
 def test_dispatch_tuning_options_match_oracle(gpu_device, oracle, opts):
     cfg = EPConfig("opts", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05)
@@ -151,12 +150,15 @@ COMBINE_CASES = [
 
 @pytest.mark.parametrize("cfg", COMBINE_CASES, ids=[c.name for c in COMBINE_CASES])
 @pytest.mark.parametrize("is_ragged", [False, True], ids=["full", "ragged"])
-@pytest.mark.parametrize("chunks,cnt", [(1, 3), (2, 3), (1, 0)])
-def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks, cnt):
+@pytest.mark.parametrize("chunks,cnt,direct", [(1, 3, 1), (2, 3, 1), (1, 0, 1), (1, 3, 0), (2, 0, 0)])
+def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks, cnt, direct):
+    """direct=1: the handle is the last dispatch's, rows come from its routing
+    state; direct=0: the general path that re-derives rows from the handle."""
     nt = ragged(cfg, is_ragged)
-    announce(f"combine {cfg} ragged={nt} chunks={chunks} nt={cnt}")
+    announce(f"combine {cfg} ragged={nt} chunks={chunks} nt={cnt} direct={direct}")
     data = generate(cfg, seed=3)
-    h = run_dispatch(cfg, data, num_tokens=nt, poison=False, options={"combine_chunks": chunks, "combine_nt": cnt})
+    h = run_dispatch(cfg, data, num_tokens=nt, poison=False,
+                     options={"combine_chunks": chunks, "combine_nt": cnt, "combine_direct": direct})
     factor = torch.arange(cfg.num_experts).float() * 0.1 + 1.0
     h.alloc_combine_io()
     h.expert_out.fill_(float("nan"))                       # rows outside the handle must never be read
@@ -181,11 +183,12 @@ def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks, cnt)
         assert bool((got[r, n:] == 7.0).all()), "rows beyond num_tokens written"
 
 
-def test_combine_skips_inactive_ranks(gpu_device, oracle):
+@pytest.mark.parametrize("direct", [1, 0])
+def test_combine_skips_inactive_ranks(gpu_device, oracle, direct):
     cfg = EPConfig("inactive", 4, 16, 1024, 16, 4, False)
-    announce("combine with an inactive rank")
+    announce(f"combine with an inactive rank direct={direct}")
     data = generate(cfg, seed=4)
-    h = run_dispatch(cfg, data, poison=False)
+    h = run_dispatch(cfg, data, poison=False, options={"combine_direct": direct})
     h.alloc_combine_io()
     h.fill_expert_out_from_recv(torch.arange(16).float() * 0.1 + 1.0)
     h.active_ranks[:, 2] = 0
@@ -196,6 +199,30 @@ def test_combine_skips_inactive_ranks(gpu_device, oracle):
                           h.layout_range.cpu(), h.num_tokens, cfg.max_tokens, cfg.num_experts,
                           active=h.active_ranks.cpu())
     assert torch.equal(h.combined.cpu().view(torch.int16), want.view(torch.int16))
+
+
+def test_combine_with_an_older_handle(gpu_device, oracle):
+    """dispatch A, dispatch B into other buffers, then combine A: the routing
+    state on the device is B's, so A's rows must be re-derived from A's handle."""
+    from mooncake_amd.harness import WorldHarness
+    cfg = EPConfig("older", 4, 24, 1024, 16, 4, False)
+    announce("combine with the handle of an older dispatch")
+    a = run_dispatch(cfg, generate(cfg, seed=7), poison=False)
+    b = WorldHarness(cfg, world=a.world)
+    b.load(generate(cfg, seed=8))
+    b.alloc_dispatch_outputs()
+    b.dispatch()
+    torch.cuda.synchronize()
+    for h, seed in ((a, 7), (b, 8)):
+        data = generate(cfg, seed=seed)
+        h.alloc_combine_io()
+        h.fill_expert_out_from_recv(torch.arange(16).float() * 0.1 + 1.0)
+        h.combine()
+        torch.cuda.synchronize()
+        want = oracle.combine(h.expert_out.cpu(), data["topk_idx"], data["topk_weights"], h.src_info.cpu(),
+                              h.layout_range.cpu(), h.num_tokens, cfg.max_tokens, cfg.num_experts)
+        # rows outside the handle hold garbage in expert_out; the oracle never reads them either
+        assert torch.equal(h.combined.cpu().view(torch.int16), want.view(torch.int16))
 
 
 def test_dispatch_with_silent_rank(gpu_device, oracle):
