@@ -51,7 +51,7 @@ struct TableChunk {
 // over units turns that into the packed row of every selection:
 //     row(sel) = ubegin[unit(sel)][expert(sel)] + selpos[sel]
 // which is the deterministic order source rank ascending, token ascending.
-constexpr int kUnitSelections = 1024;
+constexpr int kUnitSelections = 256;
 
 struct RoutingScratch {
     int32_t* ucount;     // [U, E]  selections of unit u that name expert e
@@ -132,5 +132,7 @@ hipError_t launch_fill_u32(void* dst, uint32_t value, size_t words, hipStream_t 
 // LDS the count kernel needs (per-wave counts and prefixes for every expert)
 constexpr size_t kMaxCountLdsBytes = 144 * 1024;
 size_t count_lds_bytes(const Dims& d);
+// units the prefix kernel can hold a wave's prefixes for in LDS
+constexpr int kMaxUnits = 3500;
 
 }  // namespace mcep

@@ -105,11 +105,11 @@ __device__ __forceinline__ uint64_t rank_ptr(const uint64_t* __restrict__ tbl, c
     return p.base != 0 ? p.base + (uint64_t)((int64_t)r * p.stride) : tbl[field * R + r];
 }
 
-// One block per unit (1024 consecutive (token, k) selections of one rank), one
+// One block per unit (kUnitSelections consecutive (token, k) selections of one rank), one
 // selection per thread.  Each index is read exactly once.
 //   1. inside a wave, selections naming the same expert are ranked by lane
 //      (one ballot per distinct expert present in the wave);
-//   2. the 16 waves' per-expert counts are prefix-summed in LDS, which gives
+//   2. the waves' per-expert counts are prefix-summed in LDS, which gives
 //      every selection its position inside (unit, expert) and the unit its
 //      per-expert histogram;
 // prefix_kernel then turns the units' histograms into packed-row offsets.
@@ -169,13 +169,43 @@ __global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* 
 
 // Units' histograms -> exclusive prefixes over units (source rank ascending,
 // then token ascending), recv_count, layout_range and the per-expert counts.
-// One thread per expert; the unit counts are fetched eight at a time.  (A
-// separate launch rather than "the last block of the count kernel": the
-// device-scope release that pattern needs writes back each XCD's whole L2.)
-__global__ __launch_bounds__(64) void prefix_kernel(const uint64_t* __restrict__ tbl, RoutingScratch sc, int R, int E,
-                                                     int max_tokens, int upr, int U) {
-    const int ee = blockIdx.x * blockDim.x + threadIdx.x;
+// One wave per expert, a lane per unit (64 at a time, wave-wide scan); the
+// prefixes also go to LDS, from which a lane per source rank then reads its
+// rank's begin and end.  (A separate launch rather than "the last block of the
+// count kernel": the device-scope release that pattern needs writes back each
+// XCD's whole L2, which costs more than a launch.)
+constexpr int kPrefixWaves = 4;
+
+__global__ __launch_bounds__(kPrefixWaves * 64) void prefix_kernel(const uint64_t* __restrict__ tbl,
+                                                                    RoutingScratch sc, int R, int E, int max_tokens,
+                                                                    int upr, int U) {
+    extern __shared__ int lds_prefix[];                     // [kPrefixWaves][U + 1]
+    const int lane = wave_lane();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ee = blockIdx.x * kPrefixWaves + wave;
     if (ee >= E) return;
+    int* pre = lds_prefix + (size_t)wave * (U + 1);
+    int carry = 0;
+    for (int u0 = 0; u0 < U; u0 += 64) {
+        const int u = u0 + lane;
+        const int c = (u < U) ? sc.ucount[(int64_t)u * E + ee] : 0;
+        int incl = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+        if (u < U) {
+            const int excl = carry + incl - c;
+            sc.ubegin[(int64_t)u * E + ee] = excl;
+            pre[u] = excl;
+        }
+        carry += __shfl(incl, 63);
+    }
+    if (lane == 0) pre[U] = carry;
+    // the same wave wrote pre[] and reads it below: a wave's LDS accesses complete in order
+    __builtin_amdgcn_wave_barrier();
+
     const int L = E / R;
     const int64_t RM = (int64_t)R * max_tokens;
     // A block holds RM rows.  Distinct experts per token can never exceed that;
@@ -183,37 +213,27 @@ __global__ __launch_bounds__(64) void prefix_kernel(const uint64_t* __restrict__
     const int cap = (int)(RM < 0x7fffffff ? RM : 0x7fffffff);
     const int q = ee / L, le = ee - q * L;
     const uint64_t recv_x = tbl[DF_RECV_X * R + q];       // 0: the rank takes no part and receives nothing
-    int64_t* layout_range = recv_x ? (int64_t*)tbl[DF_LAYOUT_RANGE * R + q] + (int64_t)le * R : nullptr;
-    int run = 0, rank_begin = 0;
-    for (int u0 = 0; u0 < U; u0 += 8) {
-        int cnt[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) cnt[j] = (u0 + j < U) ? sc.ucount[(int64_t)(u0 + j) * E + ee] : 0;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int uu = u0 + j;
-            if (uu >= U) break;
-            const int in_rank = uu % upr;
-            if (in_rank == 0) rank_begin = run;
-            sc.ubegin[(int64_t)uu * E + ee] = run;
-            run += cnt[j];
-            if (in_rank == upr - 1 && layout_range != nullptr) {
-                const int b = rank_begin < cap ? rank_begin : cap;
-                const int b2 = run < cap ? run : cap;
-                // count in the low half, begin in the high half; an empty pair is 0
-                layout_range[uu / upr] = (b2 > b) ? (((int64_t)b << 32) | (int64_t)(b2 - b)) : 0;
-            }
-        }
+    const int kept = carry < cap ? carry : cap;
+    if (lane == 0) {
+        sc.counts[ee] = recv_x ? kept : 0;
+        if (recv_x) ((int32_t*)tbl[DF_RECV_COUNT * R + q])[le] = kept;
     }
-    const int kept = run < cap ? run : cap;
-    sc.counts[ee] = recv_x ? kept : 0;
-    if (recv_x) ((int32_t*)tbl[DF_RECV_COUNT * R + q])[le] = kept;
+    if (recv_x == 0) return;
+    int64_t* layout_range = (int64_t*)tbl[DF_LAYOUT_RANGE * R + q] + (int64_t)le * R;
+    for (int rr = lane; rr < R; rr += 64) {
+        int b = pre[rr * upr], b2 = pre[(rr + 1) * upr];
+        b = b < cap ? b : cap;
+        b2 = b2 < cap ? b2 : cap;
+        // count in the low half, begin in the high half; an empty pair is 0
+        layout_range[rr] = (b2 > b) ? (((int64_t)b << 32) | (int64_t)(b2 - b)) : 0;
+    }
 }
 
 // The packed row of one (token, k) selection, from the routing state.
 struct SelRow {
     int e;          // global expert
     int q;          // rank that owns it
+    int le;         // its index among that rank's experts
     int64_t grow;   // row inside that rank's [L, R*max] layout: le * R*max + slot
     int slot;       // row inside the expert's block
     bool ok;
@@ -221,7 +241,7 @@ struct SelRow {
 
 __device__ __forceinline__ SelRow selection_row(const int64_t* __restrict__ idx_row, const RoutingScratch& sc, int R,
                                                 int E, int K, int max_tokens, int upr, int r, int t, int lane) {
-    SelRow s = {0, 0, 0, 0, false};
+    SelRow s = {0, 0, 0, 0, 0, false};
     if (lane < K) {
         const int i = t * K + lane;
         const int64_t e64 = idx_row[lane];
@@ -233,7 +253,8 @@ __device__ __forceinline__ SelRow selection_row(const int64_t* __restrict__ idx_
             s.slot = sc.ubegin[(int64_t)u * E + e] + pos;
             s.e = e;
             s.q = e / L;
-            s.grow = (int64_t)(e - s.q * L) * RM + s.slot;
+            s.le = e - s.q * L;
+            s.grow = (int64_t)s.le * RM + s.slot;
             s.ok = s.slot < RM;
         }
     }
@@ -267,8 +288,7 @@ __device__ __forceinline__ PackDest pack_destination(const uint64_t* __restrict_
             d.row = base + (uint64_t)s.grow * (uint64_t)H * (FP8 ? 1 : 2);
             if (FP8) {
                 const int64_t RM = (int64_t)R * max_tokens;
-                const int64_t le = s.grow / RM;   // == (grow - slot) / RM
-                d.scale = tbl[DF_RECV_SCALES * R + s.q] + (uint64_t)(le * (H / 128) * RM + s.slot) * 4;
+                d.scale = tbl[DF_RECV_SCALES * R + s.q] + (uint64_t)((int64_t)s.le * (H / 128) * RM + s.slot) * 4;
             }
             if (slab == 0) {
                 ((int32_t*)tbl[DF_SRC_INFO * R + s.q])[s.grow] = t;
@@ -505,28 +525,21 @@ __global__ __launch_bounds__(256) void scale_transpose_kernel(const uint64_t* __
         float* dp = out + row;
         int g = 0;
         if ((G & 3) == 0) {
-            constexpr int B = 8;   // 16-byte loads in flight per lane
-            for (; g + 4 * B <= G; g += 4 * B) {
+            constexpr int B = 8;   // 16-byte loads in flight per lane, also in the last, partial batch
+            for (; g < G; g += 4 * B) {
                 float4 v[B];
 #pragma unroll
-                for (int j = 0; j < B; ++j) v[j] = *(const float4*)(sp + g + 4 * j);
+                for (int j = 0; j < B; ++j)
+                    v[j] = (g + 4 * j < G) ? *(const float4*)(sp + g + 4 * j) : make_float4(0, 0, 0, 0);
                 if (valid) {
 #pragma unroll
                     for (int j = 0; j < B; ++j) {
+                        if (g + 4 * j >= G) break;
                         dp[(int64_t)(g + 4 * j + 0) * RM] = v[j].x;
                         dp[(int64_t)(g + 4 * j + 1) * RM] = v[j].y;
                         dp[(int64_t)(g + 4 * j + 2) * RM] = v[j].z;
                         dp[(int64_t)(g + 4 * j + 3) * RM] = v[j].w;
                     }
-                }
-            }
-            for (; g < G; g += 4) {
-                const float4 v = *(const float4*)(sp + g);
-                if (valid) {
-                    dp[(int64_t)(g + 0) * RM] = v.x;
-                    dp[(int64_t)(g + 1) * RM] = v.y;
-                    dp[(int64_t)(g + 2) * RM] = v.z;
-                    dp[(int64_t)(g + 3) * RM] = v.w;
                 }
             }
         }
@@ -739,8 +752,10 @@ hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const D
                        d.K, d.max_tokens, d.units_per_rank());
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
-    hipLaunchKernelGGL(prefix_kernel, dim3((d.E + 63) / 64), dim3(64), 0, stream, d_tbl, sc, d.R, d.E, d.max_tokens,
-                       d.units_per_rank(), d.units());
+    const size_t plds = (size_t)kPrefixWaves * (d.units() + 1) * sizeof(int);
+    if (plds > 60 * 1024) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(prefix_kernel, dim3((d.E + kPrefixWaves - 1) / kPrefixWaves), dim3(kPrefixWaves * 64), plds,
+                       stream, d_tbl, sc, d.R, d.E, d.max_tokens, d.units_per_rank(), d.units());
     return hipGetLastError();
 }
 

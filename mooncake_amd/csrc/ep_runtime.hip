@@ -268,6 +268,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
     // the count kernel keeps per-wave counts and prefixes of every expert in LDS
     MC_ASSERT(count_lds_bytes(d) <= kMaxCountLdsBytes);
+    MC_ASSERT(d.units() <= kMaxUnits);
     const size_t UE = (size_t)d.units() * num_experts;
     if (int rc = ensure_scratch(&w->d_ucount, &w->ucount_cap, UE)) return rc;
     if (int rc = ensure_scratch(&w->d_ubegin, &w->ubegin_cap, UE)) return rc;
