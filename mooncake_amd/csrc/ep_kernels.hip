@@ -108,7 +108,7 @@ __device__ __forceinline__ uint64_t rank_ptr(const uint64_t* __restrict__ tbl, c
 // One block per unit (kUnitSelections consecutive (token, k) selections of one rank), one
 // selection per thread.  Each index is read exactly once.
 //   1. inside a wave, selections naming the same expert are ranked by lane
-//      (one ballot per distinct expert present in the wave);
+//      (a 64-bit lane mask per expert in LDS, filled by LDS atomics);
 //   2. the waves' per-expert counts are prefix-summed in LDS, which gives
 //      every selection its position inside (unit, expert) and the unit its
 //      per-expert histogram;
@@ -119,10 +119,10 @@ __device__ __forceinline__ uint64_t rank_ptr(const uint64_t* __restrict__ tbl, c
 __global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* __restrict__ tbl, RoutingScratch sc,
                                                                  DispatchSource src, int R, int E, int K,
                                                                  int max_tokens, int upr) {
-    extern __shared__ unsigned char lds_raw[];
+    extern __shared__ unsigned long long lds_count[];
     constexpr int NW = kUnitSelections / 64;
-    uint16_t* wpre = (uint16_t*)lds_raw;                       // [NW][E] selections of e in earlier waves
-    uint8_t* wcnt = lds_raw + (size_t)NW * E * 2;              // [NW][E] selections of e in the wave
+    unsigned long long* wmask = lds_count;                     // [NW][E] lanes of the wave that name e
+    uint16_t* wpre = (uint16_t*)(lds_count + (size_t)NW * E);  // [NW][E] selections of e in earlier waves
 
     const int u = blockIdx.x;
     const int r = u / upr, c = u - r * upr;
@@ -134,37 +134,28 @@ __global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* 
 
     int64_t e64 = -1;
     if (sel < n) e64 = ((const int64_t*)rank_ptr(tbl, src.topk_idx, DF_TOPK_IDX, R, r))[sel];
-    for (int i = tid; i < NW * E / 4; i += kUnitSelections) ((uint32_t*)wcnt)[i] = 0;
+    for (int i = tid; i < NW * E; i += kUnitSelections) wmask[i] = 0;
     const bool valid = e64 >= 0 && e64 < (int64_t)E;
     const int e = valid ? (int)e64 : 0;
     __syncthreads();
 
-    int rank_in_wave = 0;
-    unsigned long long remaining = __ballot(valid);
-    while (remaining) {
-        const int leader = __builtin_ctzll(remaining);
-        const int e0 = __builtin_amdgcn_readlane(e, leader);
-        const unsigned long long m = __ballot(valid && e == e0);
-        if (valid && e == e0) {
-            rank_in_wave = __popcll(m & ((1ull << lane) - 1ull));
-            if (lane == 63 - __builtin_clzll(m)) wcnt[wave * E + e] = (uint8_t)__popcll(m);
-        }
-        remaining &= ~m;
-    }
+    // every lane sets its bit in its expert's mask; the mask then tells a lane
+    // how many lower lanes of the wave name the same expert
+    if (valid) atomicOr(&wmask[wave * E + e], 1ull << lane);
     __syncthreads();
+    const int rank_in_wave = valid ? __popcll(wmask[wave * E + e] & ((1ull << lane) - 1ull)) : 0;
 
     for (int ee = tid; ee < E; ee += kUnitSelections) {
         int run = 0;
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
             wpre[w * E + ee] = (uint16_t)run;
-            run += wcnt[w * E + ee];
+            run += __popcll(wmask[w * E + ee]);
         }
         sc.ucount[(int64_t)u * E + ee] = run;
     }
     __syncthreads();
     if (sel < n) sc.selpos[(int64_t)r * max_tokens * K + sel] = valid ? (int)wpre[wave * E + e] + rank_in_wave : -1;
-
 }
 
 // Units' histograms -> exclusive prefixes over units (source rank ascending,
@@ -736,7 +727,7 @@ hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_word
 }
 
 size_t count_lds_bytes(const Dims& d) {
-    return (size_t)(kUnitSelections / 64) * d.E * 3 + 64;
+    return (size_t)(kUnitSelections / 64) * d.E * (8 + 2) + 64;
 }
 
 hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, const Dims& d,
