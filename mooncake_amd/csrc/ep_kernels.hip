@@ -3,8 +3,8 @@
 // payload access is a 16-byte vector load or store that a wave issues over a
 // contiguous span of a row.
 //
-//   count_kernel    routing layout: per-expert histogram of every 1024-selection
-//                   unit, position of each selection inside it, exclusive
+//   count_kernel,   routing layout: per-expert histogram of every unit of 256
+//   prefix_kernel   selections, position of each selection inside it, exclusive
 //                   prefix over units, per-(expert, source rank) ranges and
 //                   per-expert counts.  Restates the count path and the slot
 //                   assignment of the reference's dispatch
@@ -16,10 +16,13 @@
 //                   quantisation with per-128 amax / 448 scales
 //                   (mooncake_ep_kernel.cu:183-186, :233-264), K row stores
 //                   straight into [local expert, R*max, hidden]
-//                   (the reference needs two hops, :273-306 then :442-466).
+//                   (the reference needs two hops, :273-306 then :442-466);
+//                   scale_transpose_kernel then moves the fp8 scales into
+//                   their column-major layout (:457-465).
 //   resolve_kernel  combine's handle (src_info, layout_range) -> source row and
 //                   weight of each (token, k) (data flow of
-//                   mooncake_ep_kernel.cu:611-637).
+//                   mooncake_ep_kernel.cu:611-637); only for a handle that is
+//                   not the last dispatch's.
 //   reduce_kernel   per token: fp32 fused multiply-add over its top-k expert
 //                   rows in k order, round to nearest even bf16
 //                   (mooncake_ep_kernel.cu:711-753).
@@ -220,35 +223,48 @@ __global__ __launch_bounds__(kPrefixWaves * 64) void prefix_kernel(const uint64_
     }
 }
 
-// The packed row of one (token, k) selection, from the routing state.
-struct SelRow {
-    int e;          // global expert
+// The packed row of one (token, k) selection, from the routing state, in two
+// steps so that callers can put their own gathers next to the one dependent
+// load (ubegin) instead of behind it: every lane works on a valid selection
+// index (lanes >= K redo lane 0's), nothing is loaded under a branch.
+struct SelKey {
+    int e;          // global expert (0 when the selection is not valid)
     int q;          // rank that owns it
     int le;         // its index among that rank's experts
-    int64_t grow;   // row inside that rank's [L, R*max] layout: le * R*max + slot
+    int pos;        // position inside (unit, expert)
+    int unit;
+    bool valid;
+};
+
+struct SelRow {
+    int64_t grow;   // row inside the owner's [L, R*max] layout: le * R*max + slot
     int slot;       // row inside the expert's block
     bool ok;
 };
 
-__device__ __forceinline__ SelRow selection_row(const int64_t* __restrict__ idx_row, const RoutingScratch& sc, int R,
+__device__ __forceinline__ SelKey selection_key(const int64_t* __restrict__ idx_row, const RoutingScratch& sc, int R,
                                                 int E, int K, int max_tokens, int upr, int r, int t, int lane) {
-    SelRow s = {0, 0, 0, 0, 0, false};
-    if (lane < K) {
-        const int i = t * K + lane;
-        const int64_t e64 = idx_row[lane];
-        const int pos = sc.selpos[(int64_t)r * max_tokens * K + i];
-        if (e64 >= 0 && e64 < (int64_t)E && pos >= 0) {
-            const int e = (int)e64, L = E / R;
-            const int u = r * upr + i / kUnitSelections;
-            const int64_t RM = (int64_t)R * max_tokens;
-            s.slot = sc.ubegin[(int64_t)u * E + e] + pos;
-            s.e = e;
-            s.q = e / L;
-            s.le = e - s.q * L;
-            s.grow = (int64_t)s.le * RM + s.slot;
-            s.ok = s.slot < RM;
-        }
-    }
+    const int li = lane < K ? lane : 0;
+    const int i = t * K + li;
+    const int64_t e64 = idx_row[li];
+    const int pos = sc.selpos[(int64_t)r * max_tokens * K + i];
+    SelKey k;
+    k.valid = lane < K && e64 >= 0 && e64 < (int64_t)E && pos >= 0;
+    k.e = k.valid ? (int)e64 : 0;
+    const int L = E / R;
+    k.q = k.e / L;
+    k.le = k.e - k.q * L;
+    k.pos = pos;
+    k.unit = r * upr + i / kUnitSelections;
+    return k;
+}
+
+__device__ __forceinline__ SelRow selection_row(const SelKey& k, int ubegin, int R, int max_tokens) {
+    const int64_t RM = (int64_t)R * max_tokens;
+    SelRow s;
+    s.slot = ubegin + k.pos;
+    s.grow = (int64_t)k.le * RM + s.slot;
+    s.ok = k.valid && s.slot < RM;
     return s;
 }
 
@@ -271,20 +287,21 @@ __device__ __forceinline__ PackDest pack_destination(const uint64_t* __restrict_
                                                      const int64_t* __restrict__ idx_row, int R, int E, int K,
                                                      int max_tokens, int H, int upr, int r, int t, int slab,
                                                      int lane) {
+    const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, upr, r, t, lane);
+    // the dependent gathers, side by side
+    const int ub = sc.ubegin[(int64_t)k.unit * E + k.e];
+    const uint64_t base = tbl[DF_RECV_X * R + k.q];
+    const uint64_t sbase = FP8 ? tbl[DF_RECV_SCALES * R + k.q] : 0;
+    const uint64_t info = (slab == 0) ? tbl[DF_SRC_INFO * R + k.q] : 0;
+    const SelRow s = selection_row(k, ub, R, max_tokens);
     PackDest d = {0, 0};
-    const SelRow s = selection_row(idx_row, sc, R, E, K, max_tokens, upr, r, t, lane);
-    if (s.ok) {
-        const uint64_t base = tbl[DF_RECV_X * R + s.q];
-        if (base != 0) {
-            d.row = base + (uint64_t)s.grow * (uint64_t)H * (FP8 ? 1 : 2);
-            if (FP8) {
-                const int64_t RM = (int64_t)R * max_tokens;
-                d.scale = tbl[DF_RECV_SCALES * R + s.q] + (uint64_t)((int64_t)s.le * (H / 128) * RM + s.slot) * 4;
-            }
-            if (slab == 0) {
-                ((int32_t*)tbl[DF_SRC_INFO * R + s.q])[s.grow] = t;
-                sc.row_src[(int64_t)s.e * R * max_tokens + s.slot] = r * max_tokens + t;
-            }
+    if (s.ok && base != 0) {
+        const int64_t RM = (int64_t)R * max_tokens;
+        d.row = base + (uint64_t)s.grow * (uint64_t)H * (FP8 ? 1 : 2);
+        if (FP8) d.scale = sbase + (uint64_t)((int64_t)k.le * (H / 128) * RM + s.slot) * 4;
+        if (slab == 0) {
+            ((int32_t*)info)[s.grow] = t;
+            sc.row_src[(int64_t)k.e * RM + s.slot] = r * max_tokens + t;
         }
     }
     return d;
@@ -626,15 +643,17 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
         if (t >= T) return;
         const int64_t* idx_row = (const int64_t*)rank_ptr(tbl, cs.topk_idx, CF_TOPK_IDX, R, r) + (int64_t)t * K;
         const float* w_row = (const float*)rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (int64_t)t * K;
-        const float wl = (lane < K) ? w_row[lane] : 0.0f;
-        const SelRow sr = selection_row(idx_row, sc, R, E, K, max_tokens, upr, r, t, lane);
-        if (sr.ok) {
-            const uint64_t base = tbl[CF_X * R + sr.q];
-            const int live = ((const int32_t*)tbl[CF_ACTIVE * R + r])[sr.q];   // skip experts on inactive ranks
-            if (base != 0 && live != 0) {
-                src = base + (uint64_t)sr.grow * (uint64_t)H * 2;
-                w = wl;
-            }
+        const float wl = w_row[lane < K ? lane : 0];
+        const int32_t* active = (const int32_t*)tbl[CF_ACTIVE * R + r];
+        const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, upr, r, t, lane);
+        // the dependent gathers, side by side
+        const int ub = sc.ubegin[(int64_t)k.unit * E + k.e];
+        const uint64_t base = tbl[CF_X * R + k.q];
+        const int live = active[k.q];                          // skip experts on inactive ranks
+        const SelRow sr = selection_row(k, ub, R, max_tokens);
+        if (sr.ok && base != 0 && live != 0) {
+            src = base + (uint64_t)sr.grow * (uint64_t)H * 2;
+            w = wl;
         }
     } else {
         // A token slot beyond the rank's count has only stale routes (zero
