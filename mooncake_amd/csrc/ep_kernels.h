@@ -104,11 +104,11 @@ struct Dims {
 struct Tuning {
     int pack_variant = 0;      // 0: 32 B/lane loads, 16 B stores; 1: two coalesced 16 B loads, 8 B stores
     int pack_waves = 4;        // waves per block in the pack kernel
-    int pack_nt = 1;           // bit 0: streaming (nontemporal) loads, bit 1: streaming stores
+    int pack_nt = -1;          // bit 0: streaming (nontemporal) loads, bit 1: streaming stores; -1: by top-k
     int uniform = 1;           // take per-rank addresses from kernel arguments when tensors are evenly spaced
     int scale_mode = 1;        // 0: scatter scales from the pack kernel; 1: staged + transposing pass
     int combine_direct = 1;    // reuse the last dispatch's routing state when combine gets that dispatch's handle
-    int combine_chunks = 1;    // 16-byte chunks per lane in the combine kernel
+    int combine_chunks = 0;    // 16-byte chunks per lane in the combine kernel (1 or 2); 0: by top-k
     int combine_waves = 4;     // waves per block in the combine kernel
     int combine_nt = 3;        // bit 0: streaming loads, bit 1: streaming stores
 };

@@ -498,61 +498,96 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
     }
 }
 
-// Staged scales -> column-major output.  kTransposeWaves waves per expert,
-// each taking 64 packed rows at a time: a lane learns its row's source token
-// slot from row_src (left by the pack kernel), reads that token's H/128 scales as
-// contiguous 16-byte pieces - a batch of them in flight at once - and stores
-// them so that the wave writes 64 consecutive floats per scale group.
-constexpr int kTransposeWaves = 8;
+// Staged scales -> column-major output.  A work item is 64 packed rows of one
+// expert times one part of kTransposeGroups scale groups, and a wave takes one
+// item: a lane learns its row's source token slot from row_src (left by the
+// pack kernel), reads that token's scales as contiguous 16-byte pieces, all in
+// flight at once, and stores them so that the wave writes 64 consecutive floats
+// per scale group.
+//
+// Which expert owns the wave's 64-row chunk follows from the per-expert row
+// counts alone: every wave scans ceil(count / 64) over the experts (a few
+// shuffles per 64 experts) and finds the expert whose chunk range holds its
+// chunk number.  The grid therefore holds no more waves than there are chunks
+// (at most one partly filled chunk per expert), however uneven the routing is.
+constexpr int kTransposeGroups = 32;      // scale groups per wave: 8 loads of 16 bytes per lane
+constexpr int kTransposeWaves = 4;        // waves per block
 
-__global__ __launch_bounds__(256) void scale_transpose_kernel(const uint64_t* __restrict__ tbl,
-                                                               const float* __restrict__ scale_stage,
-                                                               RoutingScratch scratch, int R, int E, int G,
-                                                               int max_tokens, int total_tasks) {
+__global__ __launch_bounds__(kTransposeWaves * 64) void scale_transpose_kernel(
+    const uint64_t* __restrict__ tbl, const float* __restrict__ scale_stage, RoutingScratch scratch, int R, int E,
+    int G, int max_tokens, int parts, int total_tasks) {
     const int lane = wave_lane();
-    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * kTransposeWaves + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
-    const int e = task / kTransposeWaves, wi = task - e * kTransposeWaves;
+    const int target = task / parts, part = task - target * parts;
+
+    // chunk ranges of the experts: expert e owns chunks [begin_e, begin_e + ceil(count_e / 64))
+    constexpr int kPre = 4;               // 64-expert pieces whose counts are loaded side by side
+    int pre_counts[kPre];
+#pragma unroll
+    for (int j = 0; j < kPre; ++j) {
+        const int ee = j * 64 + lane;
+        pre_counts[j] = (ee < E) ? scratch.counts[ee] : 0;
+    }
+    int carry = 0, e = -1, chunk = 0, count = 0;
+    auto piece = [&](int e0, int c) {
+        const int n = (c + 63) >> 6;
+        int incl = n;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+        const int begin = carry + incl - n;
+        const unsigned long long owns = __ballot(n > 0 && begin <= target && target < begin + n);
+        if (owns) {
+            const int l = __builtin_ctzll(owns);
+            e = e0 + l;
+            chunk = target - __shfl(begin, l);
+            count = __shfl(c, l);
+        }
+        carry += __shfl(incl, 63);
+    };
+#pragma unroll
+    for (int j = 0; j < kPre; ++j)
+        if (j * 64 < E) piece(j * 64, pre_counts[j]);
+    for (int e0 = kPre * 64; e0 < E; e0 += 64) {
+        const int ee = e0 + lane;
+        piece(e0, (ee < E) ? scratch.counts[ee] : 0);
+    }
+    if (e < 0) return;                    // beyond the last chunk
+    e = __builtin_amdgcn_readfirstlane(e);
+    chunk = __builtin_amdgcn_readfirstlane(chunk);
+    count = __builtin_amdgcn_readfirstlane(count);
+
     const int L = E / R, q = e / L, le = e - q * L;
     const int64_t RM = (int64_t)R * max_tokens;
-    // issued together: the expert's row count, this wave's first source slots
-    // (in bounds whatever the count turns out to be) and the output address
-    const int32_t* row_src = scratch.row_src + (int64_t)e * RM;
-    int row = wi * 64 + lane;
-    int slot = (row < RM) ? row_src[row] : 0;
-    const int count = scratch.counts[e];
+    const int g0 = part * kTransposeGroups;
+    const int n = (g0 + kTransposeGroups < G ? g0 + kTransposeGroups : G) - g0;
+    const int row = chunk * 64 + lane;
+    const bool valid = row < count;
+    // the output address and the row's source slot, side by side
     float* out = (float*)tbl[DF_RECV_SCALES * R + q];
-    if (wi * 64 >= count) return;
-    out += (int64_t)le * G * RM;
-
-    for (int row0 = wi * 64; row0 < count; row0 += kTransposeWaves * 64) {
-        row = row0 + lane;
-        const bool valid = row < count;
-        if (row0 != wi * 64) slot = valid ? row_src[row] : 0;
-        const float* sp = scale_stage + (int64_t)(valid ? slot : 0) * G;
-        float* dp = out + row;
-        int g = 0;
-        if ((G & 3) == 0) {
-            constexpr int B = 8;   // 16-byte loads in flight per lane, also in the last, partial batch
-            for (; g < G; g += 4 * B) {
-                float4 v[B];
+    const int slot = valid ? scratch.row_src[(int64_t)e * RM + row] : 0;
+    const float* sp = scale_stage + (int64_t)slot * G + g0;
+    float* dp = out + ((int64_t)le * G + g0) * RM + row;
+    if ((G & 3) == 0) {
+        constexpr int B = kTransposeGroups / 4;
+        float4 v[B];
 #pragma unroll
-                for (int j = 0; j < B; ++j)
-                    v[j] = (g + 4 * j < G) ? *(const float4*)(sp + g + 4 * j) : make_float4(0, 0, 0, 0);
-                if (valid) {
+        for (int j = 0; j < B; ++j) v[j] = (4 * j < n) ? *(const float4*)(sp + 4 * j) : make_float4(0, 0, 0, 0);
+        if (valid) {
 #pragma unroll
-                    for (int j = 0; j < B; ++j) {
-                        if (g + 4 * j >= G) break;
-                        dp[(int64_t)(g + 4 * j + 0) * RM] = v[j].x;
-                        dp[(int64_t)(g + 4 * j + 1) * RM] = v[j].y;
-                        dp[(int64_t)(g + 4 * j + 2) * RM] = v[j].z;
-                        dp[(int64_t)(g + 4 * j + 3) * RM] = v[j].w;
-                    }
-                }
+            for (int j = 0; j < B; ++j) {
+                if (4 * j >= n) break;
+                dp[(int64_t)(4 * j + 0) * RM] = v[j].x;
+                dp[(int64_t)(4 * j + 1) * RM] = v[j].y;
+                dp[(int64_t)(4 * j + 2) * RM] = v[j].z;
+                dp[(int64_t)(4 * j + 3) * RM] = v[j].w;
             }
         }
-        if (valid)
-            for (; g < G; ++g) dp[(int64_t)g * RM] = sp[g];
+    } else if (valid) {
+        for (int g = 0; g < n; ++g) dp[(int64_t)g * RM] = sp[g];
     }
 }
 
@@ -788,7 +823,9 @@ static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const RoutingS
 hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, float* scale_stage,
                        const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
                        hipStream_t stream) {
-    const bool ntl = t.pack_nt & 1, nts = t.pack_nt & 2;
+    // measured: streaming loads pay when a token's row goes to many experts, not when it goes to a few
+    const int pack_nt = t.pack_nt >= 0 ? t.pack_nt : (d.K > 4 ? 1 : 0);
+    const bool ntl = pack_nt & 1, nts = pack_nt & 2;
     float* stage = (use_fp8 && t.scale_mode == 1) ? scale_stage : nullptr;
     hipError_t err = hipSuccess;
     if (run_pack) {
@@ -803,10 +840,15 @@ hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const Di
 #undef MCEP_PACK
     }
     if (err != hipSuccess || stage == nullptr || !run_finish) return err;
-    const long long total = (long long)d.E * kTransposeWaves;
-    const int wpb = 4;
-    hipLaunchKernelGGL(scale_transpose_kernel, dim3((unsigned)((total + wpb - 1) / wpb)), dim3(wpb * 64), 0, stream,
-                       d_tbl, stage, sc, d.R, d.E, d.H / 128, d.max_tokens, (int)total);
+    const int G = d.H / 128;
+    const int parts = (G + kTransposeGroups - 1) / kTransposeGroups;
+    // every selection is at most one row, and each expert has at most one partly filled chunk
+    const long long chunks = ((long long)d.R * d.Tgrid * d.K + 63) / 64 + d.E;
+    const long long total = chunks * parts;
+    if (total > 0x7fffffffll) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(scale_transpose_kernel, dim3((unsigned)((total + kTransposeWaves - 1) / kTransposeWaves)),
+                       dim3(kTransposeWaves * 64), 0, stream, d_tbl, stage, sc, d.R, d.E, G, d.max_tokens, parts,
+                       (int)total);
     return hipGetLastError();
 }
 
@@ -858,7 +900,8 @@ hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, ui
                          bool direct, const CombineSource& src, const void* d_zero_row, const Dims& d, const Tuning& t,
                          hipStream_t stream) {
     const ReduceLaunch rl{d_tbl, d_routes, stamp, sc, src, d_zero_row};
-    const int ch = t.combine_chunks >= 2 ? 2 : 1;
+    // measured: with few rows per token a lane needs two chunks to keep enough loads in flight
+    const int ch = t.combine_chunks > 0 ? (t.combine_chunks >= 2 ? 2 : 1) : (d.K <= 4 ? 2 : 1);
 #define MCEP_K(KMAX)                                                                                   \
     do {                                                                                               \
         if (direct) return ch == 2 ? launch_reduce_t<KMAX, 2, true>(rl, d, t, stream)                  \
