@@ -109,6 +109,53 @@ int mc_ep_world_combine(mc_ep_world_t* world, const uint64_t* x_ptrs, const uint
                         int num_max_dispatch_tokens_per_rank, int num_experts, const uint64_t* combined_x_ptrs,
                         int phases, uint64_t stream_ptr);
 
+/* ---- the native benchmark loop ------------------------------------------ */
+
+/* _benchmark_legacy_buffer (bound in mooncake-ep/src/ep_py.cpp:12,26; the loop
+ * is mooncake-ep/benchmarks/legacy_buffer_perf.cpp:84-146): clear
+ * packed_recv_count, bf16 dispatch, combine, repeated `warmups` times untimed
+ * and `iterations` times between a pair of events each; the first timed
+ * iteration is dropped.  The structs are LegacyBufferPerfTensors / Config /
+ * Result (legacy_buffer_perf.cpp:18-49) with one device address per logical
+ * rank where the reference has one address: the loop drives the whole world,
+ * every rank with num_tokens tokens.  A null address or a configuration the
+ * reference's validate() rejects (:58-82) gives MC_EP_ERR_ASSERT with the
+ * reference's message. */
+typedef struct {
+    const uint64_t* x_ptrs;                          /* [T, H] bf16 */
+    const uint64_t* topk_idx_ptrs;                   /* [T, K] int64 */
+    const uint64_t* topk_weights_ptrs;               /* [T, K] f32 */
+    const uint64_t* active_ranks_ptrs;               /* [R] int32 */
+    const uint64_t* expert_x_ptrs;                   /* [E/R, R*max, H] bf16: what combine reads */
+    const uint64_t* packed_recv_x_ptrs;              /* [E/R, R*max, H] bf16 */
+    const uint64_t* packed_recv_count_ptrs;          /* [E/R] int32 */
+    const uint64_t* packed_recv_src_info_ptrs;       /* [E/R, R*max] int32 */
+    const uint64_t* packed_recv_layout_range_ptrs;   /* [E/R, R] int64 */
+    const uint64_t* combined_x_ptrs;                 /* [T, H] bf16 */
+} mc_ep_legacy_perf_tensors_t;
+
+typedef struct {
+    int num_tokens;
+    int hidden;
+    int num_topk;
+    int num_local_experts;
+    int num_max_dispatch_tokens_per_rank;
+    int num_experts;
+    int timeout_us;                                  /* -1; kept for the reference's layout, unused */
+    int warmups;                                     /* reference default 20 */
+    int iterations;                                  /* reference default 30; > 1 */
+    uint64_t compute_stream_ptr;
+} mc_ep_legacy_perf_config_t;
+
+typedef struct {
+    double average_us;
+    double min_us;
+    double max_us;
+} mc_ep_legacy_perf_result_t;
+
+int mc_ep_world_legacy_buffer_perf(mc_ep_world_t* world, const mc_ep_legacy_perf_tensors_t* tensors,
+                                   const mc_ep_legacy_perf_config_t* config, mc_ep_legacy_perf_result_t* result);
+
 /* ---- per-rank Buffer: the reference's binding, one object per rank ------ */
 
 /* MooncakeEpBuffer(rank, num_ranks, num_ep_buffer_bytes, disable_p2p),

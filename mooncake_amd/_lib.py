@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_uint64, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_double, c_int, c_int32, c_int64, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmooncake_ep_hip.so")
@@ -20,6 +20,27 @@ _lib = None
 _U64P = POINTER(c_uint64)
 _I32P = POINTER(c_int32)
 _VPP = POINTER(c_void_p)
+
+
+
+class LegacyPerfTensors(Structure):
+    """mc_ep_legacy_perf_tensors_t: one array of per-rank device addresses per tensor."""
+    _fields_ = [(name, _U64P) for name in (
+        "x_ptrs", "topk_idx_ptrs", "topk_weights_ptrs", "active_ranks_ptrs", "expert_x_ptrs", "packed_recv_x_ptrs",
+        "packed_recv_count_ptrs", "packed_recv_src_info_ptrs", "packed_recv_layout_range_ptrs", "combined_x_ptrs")]
+
+
+class LegacyPerfConfig(Structure):
+    """mc_ep_legacy_perf_config_t"""
+    _fields_ = [(name, c_int) for name in (
+        "num_tokens", "hidden", "num_topk", "num_local_experts", "num_max_dispatch_tokens_per_rank", "num_experts",
+        "timeout_us", "warmups", "iterations")] + [("compute_stream_ptr", c_uint64)]
+
+
+class LegacyPerfResult(Structure):
+    """mc_ep_legacy_perf_result_t"""
+    _fields_ = [("average_us", c_double), ("min_us", c_double), ("max_us", c_double)]
+
 
 # name -> (restype, argtypes); one entry per declaration in include/mooncake_ep_hip.h
 SIGNATURES = {
@@ -35,6 +56,8 @@ SIGNATURES = {
                                      _U64P, _U64P, _U64P, _U64P, _U64P, c_int, c_uint64]),
     "mc_ep_world_combine": (c_int, [c_void_p, _U64P, _U64P, _U64P, _U64P, _U64P, _U64P, _I32P, c_int, c_int,
                                     c_int, c_int, _U64P, c_int, c_uint64]),
+    "mc_ep_world_legacy_buffer_perf": (c_int, [c_void_p, POINTER(LegacyPerfTensors), POINTER(LegacyPerfConfig),
+                                               POINTER(LegacyPerfResult)]),
     "mc_ep_buffer_create": (c_int, [c_void_p, c_int, c_int64, c_int, _VPP]),
     "mc_ep_buffer_destroy": (c_int, [c_void_p]),
     "mc_ep_buffer_ibgda_disabled": (c_int, [c_void_p]),

@@ -127,6 +127,8 @@ hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, ui
                          bool direct, const CombineSource& src, const void* d_zero_row, const Dims& d, const Tuning& t,
                          hipStream_t stream);
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
+// zero `words` 32-bit words at each of n_ptrs device addresses (host array), one launch per kTableChunk addresses
+hipError_t launch_clear_words(const uint64_t* h_ptrs, int n_ptrs, int words, hipStream_t stream);
 hipError_t launch_fill_u32(void* dst, uint32_t value, size_t words, hipStream_t stream);
 
 // LDS the count kernel needs (per-wave counts and prefixes for every expert)

@@ -100,6 +100,13 @@ __global__ void table_write_kernel(uint64_t* dst, TableChunk chunk, int n) {
     if (i < n) dst[i] = chunk.v[i];
 }
 
+// Clears `words` 32-bit words at each of n addresses carried in kernel
+// arguments: one launch where a per-rank hipMemsetAsync would be n launches.
+__global__ void clear_words_kernel(TableChunk chunk, int n, int words) {
+    const int i = threadIdx.x + blockIdx.x * blockDim.x;
+    if (i < n * words) ((uint32_t*)chunk.v[i / words])[i % words] = 0u;
+}
+
 // ---------------------------------------------------------------------------
 // routing layout
 // ---------------------------------------------------------------------------
@@ -774,6 +781,22 @@ hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_word
         for (int i = 0; i < n; ++i) chunk.v[i] = h_tbl[base + i];
         for (int i = n; i < kTableChunk; ++i) chunk.v[i] = 0;
         hipLaunchKernelGGL(table_write_kernel, dim3((n + 127) / 128), dim3(128), 0, stream, d_tbl + base, chunk, n);
+        hipError_t err = hipGetLastError();
+        if (err != hipSuccess) return err;
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_clear_words(const uint64_t* h_ptrs, int n_ptrs, int words, hipStream_t stream) {
+    if (words <= 0) return hipSuccess;
+    TableChunk chunk;
+    for (int base = 0; base < n_ptrs; base += kTableChunk) {
+        const int n = (n_ptrs - base < kTableChunk) ? (n_ptrs - base) : kTableChunk;
+        for (int i = 0; i < kTableChunk; ++i) chunk.v[i] = i < n ? h_ptrs[base + i] : 0;
+        const long long total = (long long)n * words;
+        if (total > 0x7fffffffll) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, chunk, n,
+                           words);
         hipError_t err = hipGetLastError();
         if (err != hipSuccess) return err;
     }

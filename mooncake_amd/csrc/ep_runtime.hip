@@ -681,6 +681,91 @@ int mc_ep_world_combine(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_t
                               combined_x_ptrs, phases, (hipStream_t)stream_ptr);
 }
 
+int mc_ep_world_legacy_buffer_perf(mc_ep_world_t* w, const mc_ep_legacy_perf_tensors_t* t,
+                                   const mc_ep_legacy_perf_config_t* c, mc_ep_legacy_perf_result_t* result) {
+    MC_ASSERT(w != nullptr && t != nullptr && c != nullptr && result != nullptr);
+    if (c->num_tokens <= 0 || c->hidden <= 0 || c->num_topk <= 0 ||
+        c->num_max_dispatch_tokens_per_rank < c->num_tokens || c->num_experts <= 0 || c->num_local_experts <= 0 ||
+        c->warmups < 0 || c->iterations <= 1)
+        return fail(MC_EP_ERR_ASSERT, "invalid legacy EP benchmark configuration");
+    const uint64_t* const fields[] = {t->x_ptrs,
+                                      t->topk_idx_ptrs,
+                                      t->topk_weights_ptrs,
+                                      t->active_ranks_ptrs,
+                                      t->expert_x_ptrs,
+                                      t->packed_recv_x_ptrs,
+                                      t->packed_recv_count_ptrs,
+                                      t->packed_recv_src_info_ptrs,
+                                      t->packed_recv_layout_range_ptrs,
+                                      t->combined_x_ptrs};
+    for (const uint64_t* f : fields) {
+        if (f == nullptr) return fail(MC_EP_ERR_ASSERT, "legacy EP benchmark received a null tensor pointer");
+        for (int r = 0; r < w->R; ++r)
+            if (f[r] == 0) return fail(MC_EP_ERR_ASSERT, "legacy EP benchmark received a null tensor pointer");
+    }
+    MC_ASSERT(c->num_local_experts * w->R == c->num_experts);
+
+    DeviceGuard guard(w->device);
+    hipStream_t stream = (hipStream_t)c->compute_stream_ptr;
+    const std::vector<int32_t> tokens((size_t)w->R, c->num_tokens);
+
+    auto run_once = [&]() -> int {
+        // the reference's cudaMemsetAsync(packed_recv_count) of every rank, in one launch
+        MC_HIP(launch_clear_words(t->packed_recv_count_ptrs, w->R, c->num_local_experts, stream));
+        int rc = world_dispatch_impl(w, t->x_ptrs, t->topk_idx_ptrs, tokens.data(), c->hidden, c->num_topk,
+                                     c->num_max_dispatch_tokens_per_rank, c->num_experts, 0, t->packed_recv_x_ptrs,
+                                     nullptr, t->packed_recv_count_ptrs, t->packed_recv_src_info_ptrs,
+                                     t->packed_recv_layout_range_ptrs, MC_EP_PHASE_ALL, stream);
+        if (rc != MC_EP_OK) return rc;
+        return world_combine_impl(w, t->expert_x_ptrs, t->topk_idx_ptrs, t->topk_weights_ptrs,
+                                  t->packed_recv_src_info_ptrs, t->packed_recv_layout_range_ptrs,
+                                  t->active_ranks_ptrs, tokens.data(), c->hidden, c->num_topk,
+                                  c->num_max_dispatch_tokens_per_rank, c->num_experts, t->combined_x_ptrs,
+                                  MC_EP_PHASE_ALL, stream);
+    };
+
+    for (int i = 0; i < c->warmups; ++i) {
+        const int rc = run_once();
+        if (rc != MC_EP_OK) return rc;
+    }
+    MC_HIP(hipStreamSynchronize(stream));
+
+    // events are released on every way out
+    struct Events {
+        std::vector<hipEvent_t> v;
+        ~Events() {
+            for (hipEvent_t e : v) (void)hipEventDestroy(e);
+        }
+    } starts, ends;
+    for (int i = 0; i < c->iterations; ++i) {
+        hipEvent_t s = nullptr, e = nullptr;
+        MC_HIP(hipEventCreate(&s));
+        starts.v.push_back(s);
+        MC_HIP(hipEventCreate(&e));
+        ends.v.push_back(e);
+        MC_HIP(hipEventRecord(s, stream));
+        const int rc = run_once();
+        if (rc != MC_EP_OK) return rc;
+        MC_HIP(hipEventRecord(e, stream));
+    }
+    MC_HIP(hipEventSynchronize(ends.v.back()));
+
+    // the first timed iteration is dropped, as in the reference
+    double total = 0.0, lo = 0.0, hi = 0.0;
+    for (int i = 1; i < c->iterations; ++i) {
+        float ms = 0.0f;
+        MC_HIP(hipEventElapsedTime(&ms, starts.v[i], ends.v[i]));
+        const double us = (double)ms * 1000.0;
+        total += us;
+        if (i == 1 || us < lo) lo = us;
+        if (i == 1 || us > hi) hi = us;
+    }
+    result->average_us = total / (c->iterations - 1);
+    result->min_us = lo;
+    result->max_us = hi;
+    return MC_EP_OK;
+}
+
 int mc_ep_buffer_create(mc_ep_world_t* w, int rank, int64_t num_ep_buffer_bytes, int disable_p2p,
                         mc_ep_buffer_t** out) {
     MC_ASSERT(w != nullptr && out != nullptr);

@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_void_p
-from typing import Callable, Dict, List, Optional, Tuple
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 from . import _lib
 
@@ -103,6 +103,30 @@ class World:
         self.prepare_combine(x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
                              active_ranks_ptrs, num_combined_tokens, hidden, num_topk,
                              num_max_dispatch_tokens_per_rank, num_experts, combined_x_ptrs)(stream_ptr, phases)
+
+
+    def legacy_buffer_perf(self, tensors: Dict[str, Sequence[int]], num_tokens: int, hidden: int, num_topk: int,
+                           num_local_experts: int, num_max_dispatch_tokens_per_rank: int, num_experts: int,
+                           warmups: int = 20, iterations: int = 30, timeout_us: int = -1,
+                           compute_stream_ptr: int = 0) -> Tuple[float, float, float]:
+        """The native loop `mooncake._ep._benchmark_legacy_buffer` runs
+        (mooncake-ep/benchmarks/legacy_buffer_perf.cpp:84-146), over the whole
+        world: returns (average_us, min_us, max_us) of recv_count clear + bf16
+        dispatch + combine.  `tensors` maps the field names of
+        LegacyBufferPerfTensors (x_ptr -> "x", ...) to per-rank addresses."""
+        t = _lib.LegacyPerfTensors()
+        keep = []
+        for field, _ in _lib.LegacyPerfTensors._fields_:
+            values = tensors.get(field[:-len("_ptrs")])
+            arr = _lib.u64_array(values) if values is not None else None
+            keep.append(arr)
+            setattr(t, field, arr)
+        c = _lib.LegacyPerfConfig(num_tokens, hidden, num_topk, num_local_experts, num_max_dispatch_tokens_per_rank,
+                                  num_experts, timeout_us, warmups, iterations, compute_stream_ptr)
+        r = _lib.LegacyPerfResult()
+        _lib.check(_lib.lib().mc_ep_world_legacy_buffer_perf(self._h, ctypes.byref(t), ctypes.byref(c),
+                                                             ctypes.byref(r)))
+        return r.average_us, r.min_us, r.max_us
 
 
 _default_worlds: Dict[int, World] = {}

@@ -81,9 +81,11 @@ class Buffer:
         self.runtime = ep.Buffer(self.rank, self.group_size, num_ep_buffer_bytes, disable_p2p, world=world)
         # there is no slow path here: the HIP kernels are the only implementation
         self._use_fallback = False
-        # a round may be launched by a later rank's call: keep the tensors of
-        # recent calls alive until then
-        self._keepalive = collections.deque(maxlen=32)
+        # a round is launched by its last rank's call, which comes before this
+        # rank's next call of the same kind: keeping the tensors of the last
+        # two dispatches and combines alive covers it (a longer history would
+        # pin gigabytes of packed buffers per rank)
+        self._keepalive = collections.deque(maxlen=4)
         self.connect()
 
     def connect(self, active_ranks=None) -> None:
