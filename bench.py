@@ -143,7 +143,7 @@ def main():
     h.alloc_dispatch_outputs()
     h.alloc_combine_io()
     h.dispatch()
-    h.fill_expert_out_from_recv()          # expert outputs = dequantised dispatched rows
+    h.cast_back()                          # expert outputs = dispatched rows cast back to bf16 (consumer kernel)
     torch.cuda.synchronize()
 
     def step():
@@ -169,6 +169,19 @@ def main():
     kernels = {k: {"us": round(v[0], 2), "min_us": round(v[1], 2)} for k, v in t.items()}
     kernels["pack"].update(bytes=alg["dispatch"], GBps=round(alg["dispatch"] / pack_us / 1e3, 1))
     kernels["reduce"].update(bytes=alg["combine"], GBps=round(alg["combine"] / red_us / 1e3, 1))
+    # the consumer of the packed layout (valid rows -> bf16), outside the step: reported, not part of `value`
+    H = cfg.hidden
+    cast_bytes = S * ((H + H // 128 * 4) if cfg.use_fp8 else 2 * H) + S * 2 * H
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.kernel_iters + 1)]
+    for _ in range(3):
+        h.cast_back()
+    for i in range(args.kernel_iters):
+        ev[i].record()
+        h.cast_back()
+    ev[-1].record()
+    torch.cuda.synchronize()
+    cast_us = ev[0].elapsed_time(ev[-1]) / args.kernel_iters * 1e3
+    consumer = {"cast_back_us": round(cast_us, 2), "bytes": cast_bytes, "GBps": round(cast_bytes / cast_us / 1e3, 1)}
     # the dominant kernel is the one the step spends most time in
     dom = "reduce" if red_us >= pack_us else "pack"
     achieved = kernels[dom]["GBps"]
@@ -194,6 +207,7 @@ def main():
         "tokens_per_s": round(cfg.total_tokens / ((d_us + c_us) * 1e-6), 1),
         "algorithmic_bytes": alg,
         "kernels": kernels,
+        "consumer": consumer,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get((cfg.name, dom)) if not opts else None},

@@ -109,6 +109,24 @@ int mc_ep_world_combine(mc_ep_world_t* world, const uint64_t* x_ptrs, const uint
                         int num_max_dispatch_tokens_per_rank, int num_experts, const uint64_t* combined_x_ptrs,
                         int phases, uint64_t stream_ptr);
 
+/* ---- consumer of the packed layout --------------------------------------- */
+
+/* What the reference's callers do with dispatch's output before the expert
+ * GEMMs: per_token_cast_back (mooncake-wheel/tests/ep_test_utils.py:50-53) /
+ * dequantize_fp8 (mooncake-ep/tests/test_ep_grid.py:43-48): bf16(f32(fp8) *
+ * scale) per 128-element group, reading the scales in the column-major layout
+ * dispatch writes (mooncake_ep_buffer.py:479-487) - and, when
+ * expert_factor_ptr != 0 (device f32 [num_experts]), the grid test's mock
+ * expert on top, bf16(row * factor[expert]) (test_ep_grid.py:168-173).  Only
+ * rows below packed_recv_count are read or written.  packed_recv_x_scales_ptrs
+ * == NULL means the payload is bf16 (then only the factor applies; out may
+ * alias the input).  num_topk bounds the number of valid rows (at most one per
+ * selection); 0 if unknown.  Out: [E/R, R*max, hidden] bf16 per rank. */
+int mc_ep_world_cast_back(mc_ep_world_t* world, const uint64_t* packed_recv_x_ptrs,
+                          const uint64_t* packed_recv_x_scales_ptrs, const uint64_t* packed_recv_count_ptrs,
+                          uint64_t expert_factor_ptr, const uint64_t* out_ptrs, int hidden, int num_topk,
+                          int num_max_dispatch_tokens_per_rank, int num_experts, uint64_t stream_ptr);
+
 /* ---- the native benchmark loop ------------------------------------------ */
 
 /* _benchmark_legacy_buffer (bound in mooncake-ep/src/ep_py.cpp:12,26; the loop

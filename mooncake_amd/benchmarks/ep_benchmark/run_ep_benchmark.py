@@ -198,7 +198,7 @@ class EPBenchmark:
             mark(0)
             self.harness.dispatch()
             mark(1)
-            self.harness.fill_expert_out_from_recv(self.factor)
+            self.harness.cast_back(self.factor)     # the mock expert, valid rows only, by the consumer kernel
             mark(2)
             self.harness.combine()
             mark(3)

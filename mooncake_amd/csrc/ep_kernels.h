@@ -35,6 +35,15 @@ enum CombineField : int {
     CF_COUNT
 };
 
+// table of the packed layout's consumer (cast back to bf16)
+enum ConsumerField : int {
+    XF_RECV_X = 0,     // const fp8|bf16* [L, R*max, H]   (0: rank takes no part)
+    XF_RECV_SCALES,    // const float*    [L, H/128, R*max] (fp8 only)
+    XF_RECV_COUNT,     // const int32*    [L]
+    XF_OUT,            // bf16*           [L, R*max, H]
+    XF_COUNT
+};
+
 constexpr int kMaxTopK = 16;          // the reference caps top-k at 11 (mooncake_ep_kernel.cu:487,773)
 constexpr int kTableChunk = 384;      // table words one writer launch carries in its kernel arguments
 constexpr size_t kZeroRowBytes = 64 * 1024;   // zero row that masked selections read: hidden <= 32768
@@ -126,6 +135,11 @@ hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_
 hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const RoutingScratch& sc,
                          bool direct, const CombineSource& src, const void* d_zero_row, const Dims& d, const Tuning& t,
                          hipStream_t stream);
+// packed rows below packed_recv_count -> bf16 rows times factor[expert]; max_rows bounds the world's valid rows
+// d_chunk_map: 16 bytes x (cast_back_chunks(max_rows, E) + 1) of scratch for the kernel's work list
+long long cast_back_chunks(long long max_rows, int num_experts);
+hipError_t launch_cast_back(const uint64_t* d_tbl, void* d_chunk_map, const float* d_factor, bool use_fp8,
+                            long long max_rows, const Dims& d, hipStream_t stream);
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 // zero `words` 32-bit words at each of n_ptrs device addresses (host array), one launch per kTableChunk addresses
 hipError_t launch_clear_words(const uint64_t* h_ptrs, int n_ptrs, int words, hipStream_t stream);

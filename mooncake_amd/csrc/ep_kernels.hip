@@ -756,6 +756,183 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
     }
 }
 
+// ---------------------------------------------------------------------------
+// consumer of the packed layout: cast back to bf16 (+ per-expert factor)
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 pr = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf2));   // v_cvt_pk_bf16_f32
+}
+
+// out = bf16(bf16(a * s) * f), both roundings to nearest even, for a pair
+__device__ __forceinline__ uint32_t scale_round_twice(float a, float b, float s, float f) {
+    const uint32_t once = pack_bf16_rne(a * s, b * s);
+    return pack_bf16_rne(bf16_lo(once) * f, bf16_hi(once) * f);
+}
+
+// Work list of the cast-back kernel: which (expert, row chunk) each chunk
+// number is, from the packed_recv_count tensors alone; map[0].x is the number
+// of chunks.  Per block: a thread per expert fetches the count, one wave scans
+// ceil(count / kCastRows) over the experts in LDS, then a thread per chunk
+// finds its expert by bisection of the scanned begins.  It costs a launch, and
+// saves every block of the main kernel the same scan (a chain of dependent
+// loads) in front of its first row.
+constexpr int kCastRows = 4;
+constexpr int kCastCols = 1024;
+constexpr int kCastMaxExperts = 4096;
+constexpr int kCastMapBlocks = 8;      // each repeats the scan (cheap) and writes an eighth of the entries
+
+__global__ __launch_bounds__(1024) void cast_chunks_kernel(const uint64_t* __restrict__ tbl, int4* __restrict__ map,
+                                                           int R, int E, int max_tokens, int max_chunks) {
+    __shared__ int lds_count[kCastMaxExperts];
+    __shared__ int lds_begin[kCastMaxExperts + 1];
+    const int lane = wave_lane();
+    const int L = E / R;
+    const int64_t RM = (int64_t)R * max_tokens;
+    for (int ee = threadIdx.x; ee < E; ee += blockDim.x) {
+        const int qq = ee / L;
+        const int32_t* cnt = (const int32_t*)tbl[XF_RECV_COUNT * R + qq];
+        int c = 0;
+        // a rank without tensors takes no part
+        if (cnt != nullptr && tbl[XF_RECV_X * R + qq] != 0 && tbl[XF_OUT * R + qq] != 0) c = cnt[ee - qq * L];
+        lds_count[ee] = c < 0 ? 0 : (c > RM ? (int)RM : c);
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        int carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int ee = e0 + lane;
+            const int n = (ee < E) ? (lds_count[ee] + kCastRows - 1) / kCastRows : 0;
+            int incl = n;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int up = __shfl_up(incl, d);
+                if (lane >= d) incl += up;
+            }
+            if (ee < E) lds_begin[ee] = carry + incl - n;
+            carry += __shfl(incl, 63);
+        }
+        if (lane == 0) {
+            lds_begin[E] = carry;
+            if (blockIdx.x == 0) map[0] = make_int4(carry < max_chunks ? carry : max_chunks, 0, 0, 0);
+        }
+    }
+    __syncthreads();
+    const int total = lds_begin[E] < max_chunks ? lds_begin[E] : max_chunks;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        // the last expert whose first chunk number is <= i (experts without rows share their successor's begin)
+        int lo = 0, hi = E;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (lds_begin[mid] <= i) lo = mid; else hi = mid;
+        }
+        map[1 + i] = make_int4(lo, i - lds_begin[lo], lds_count[lo], 0);
+    }
+}
+
+// A block takes one chunk (kCastRows consecutive packed rows of one expert)
+// times kCastCols columns, so only rows below packed_recv_count cost anything.
+// The chunk's scales (column-major in memory: 64 consecutive rows of one group
+// are 256 contiguous bytes) are staged in LDS; then each wave converts its 16
+// rows, 16 payload bytes (FP8) or 32 (bf16 payload) per lane and row.
+template <bool FP8>
+__global__ __launch_bounds__(256) void cast_back_kernel(const uint64_t* __restrict__ tbl,
+                                                         const int4* __restrict__ map,
+                                                         const float* __restrict__ factor, int R, int E, int H,
+                                                         int max_tokens, int parts) {
+    const int lane = wave_lane();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int target = blockIdx.x / parts, part = blockIdx.x - target * parts;
+    const int L = E / R;
+    const int64_t RM = (int64_t)R * max_tokens;
+    const int total = map[0].x;
+    const int4 item = map[1 + target];      // in bounds: the map holds an entry per possible chunk
+    if (target >= total) return;            // block-uniform
+    const int e = __builtin_amdgcn_readfirstlane(item.x);
+    const int chunk = __builtin_amdgcn_readfirstlane(item.y);
+    const int count = __builtin_amdgcn_readfirstlane(item.z);
+
+    const int q = e / L, le = e - q * L;
+    const int G = H / 128;
+    const int col0 = part * kCastCols;
+    const int ncols = (H - col0 < kCastCols) ? (H - col0) : kCastCols;
+    const int row0 = chunk * kCastRows;
+    const float f = factor != nullptr ? factor[e] : 1.0f;
+    const uint8_t* in = (const uint8_t*)tbl[XF_RECV_X * R + q];
+    uint8_t* out = (uint8_t*)tbl[XF_OUT * R + q];
+
+    // A lane owns two pieces of 8 elements, half a block's width apart, so that each
+    // of its two 16-byte stores lands in a run of 1 KB written by the wave as a whole.
+    // Piece p covers columns col0 + p * 512 + lane * 8 .. + 7; 16 lanes share a scale group.
+    constexpr int kHalf = kCastCols / 2;
+    constexpr int kIn = FP8 ? 8 : 16;               // payload bytes per piece
+    bool on[2];
+    int64_t in_off[2], out_off[2];
+    const float* scale_col[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int col = p * kHalf + lane * 8;
+        on[p] = col < ncols;
+        const int c = on[p] ? col : 0;
+        in_off[p] = (int64_t)(col0 + c) * (FP8 ? 1 : 2);
+        out_off[p] = (int64_t)(col0 + c) * 2;
+        scale_col[p] = FP8 ? (const float*)tbl[XF_RECV_SCALES * R + q] + ((int64_t)le * G + (col0 + c) / 128) * RM
+                           : nullptr;
+    }
+
+    constexpr int kBatch = kCastRows / 4 < 8 ? kCastRows / 4 : 8;   // rows whose loads are in flight together
+    const int64_t row_base = (int64_t)le * RM;
+    for (int b = 0; b < kCastRows / 4; b += kBatch) {
+        const int r_first = row0 + wave * (kCastRows / 4) + b;
+        if (r_first >= count) break;
+        uint4 v[kBatch][2];
+        float sv[kBatch][2];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const int row = r_first + i < count ? r_first + i : r_first;
+            const uint8_t* src = in + (row_base + row) * H * (FP8 ? 1 : 2);
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                if (FP8) {
+                    const uint2 w = *(const uint2*)(src + in_off[p]);
+                    v[i][p] = make_uint4(w.x, w.y, 0u, 0u);
+                    sv[i][p] = scale_col[p][row];
+                } else {
+                    v[i][p] = load16<true>(src + in_off[p]);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            if (r_first + i >= count) break;       // wave-uniform
+            uint8_t* dst = out + (row_base + r_first + i) * H * 2;
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                uint32_t o[4];
+                if (FP8) {
+                    typedef float f2 __attribute__((ext_vector_type(2)));
+                    const f2 a0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[i][p].x, false);
+                    const f2 a1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[i][p].x, true);
+                    const f2 a2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[i][p].y, false);
+                    const f2 a3 = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[i][p].y, true);
+                    const float sc = sv[i][p];
+                    o[0] = scale_round_twice(a0.x, a0.y, sc, f);
+                    o[1] = scale_round_twice(a1.x, a1.y, sc, f);
+                    o[2] = scale_round_twice(a2.x, a2.y, sc, f);
+                    o[3] = scale_round_twice(a3.x, a3.y, sc, f);
+                } else {
+                    const uint32_t w[4] = {v[i][p].x, v[i][p].y, v[i][p].z, v[i][p].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) o[j] = pack_bf16_rne(bf16_lo(w[j]) * f, bf16_hi(w[j]) * f);
+                }
+                if (on[p]) store16<false>(dst + out_off[p], make_uint4(o[0], o[1], o[2], o[3]));
+            }
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -940,6 +1117,30 @@ hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, ui
     if (d.K <= 12) MCEP_K(12);
     MCEP_K(16);
 #undef MCEP_K
+}
+
+long long cast_back_chunks(long long max_rows, int num_experts) {
+    // every row is in one chunk, and each expert has at most one partly filled chunk
+    return (max_rows + kCastRows - 1) / kCastRows + num_experts;
+}
+
+hipError_t launch_cast_back(const uint64_t* d_tbl, void* d_chunk_map, const float* d_factor, bool use_fp8,
+                            long long max_rows, const Dims& d, hipStream_t stream) {
+    const int parts = (d.H + kCastCols - 1) / kCastCols;
+    const long long chunks = cast_back_chunks(max_rows, d.E);
+    const long long total = chunks * parts;
+    if (total <= 0) return hipSuccess;
+    if (total > 0x7fffffffll || d.E > kCastMaxExperts) return hipErrorInvalidValue;
+    int4* map = (int4*)d_chunk_map;
+    hipLaunchKernelGGL(cast_chunks_kernel, dim3(kCastMapBlocks), dim3(1024), 0, stream, d_tbl, map, d.R, d.E, d.max_tokens,
+                       (int)chunks);
+    if (use_fp8)
+        hipLaunchKernelGGL(cast_back_kernel<true>, dim3((unsigned)total), dim3(256), 0, stream, d_tbl, map, d_factor,
+                           d.R, d.E, d.H, d.max_tokens, parts);
+    else
+        hipLaunchKernelGGL(cast_back_kernel<false>, dim3((unsigned)total), dim3(256), 0, stream, d_tbl, map, d_factor,
+                           d.R, d.E, d.H, d.max_tokens, parts);
+    return hipGetLastError();
 }
 
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t stream) {

@@ -81,8 +81,8 @@ struct mc_ep_world {
     int device = 0;
     int R = 0;
     hipStream_t comm_stream = nullptr;
-    uint64_t* d_tbl[2] = {nullptr, nullptr};     // dispatch, combine pointer tables
-    std::vector<uint64_t> tbl_cache[2];           // what the device tables hold
+    uint64_t* d_tbl[3] = {nullptr, nullptr, nullptr};   // dispatch, combine, consumer pointer tables
+    std::vector<uint64_t> tbl_cache[3];                  // what the device tables hold
     // routing state of the last dispatch (see RoutingScratch)
     int32_t* d_ucount = nullptr;
     size_t ucount_cap = 0;
@@ -96,6 +96,8 @@ struct mc_ep_world {
     size_t counts_cap = 0;
     uint32_t* d_ticket = nullptr;
     size_t ticket_cap = 0;
+    uint32_t* d_chunk_map = nullptr;     // work list of the cast-back kernel, 4 words per entry
+    size_t chunk_map_cap = 0;
     // what the last dispatch was called with, so that a combine given that
     // dispatch's handle can reuse its routing state instead of re-deriving rows
     struct LastDispatch {
@@ -586,8 +588,9 @@ int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
     w->R = num_ranks;
     MC_HIP(hipGetDevice(&w->device));
     MC_HIP(hipStreamCreateWithFlags(&w->comm_stream, hipStreamNonBlocking));
-    for (int i = 0; i < 2; ++i) {
-        const size_t words = (size_t)(i == 0 ? (int)DF_COUNT : (int)CF_COUNT) * num_ranks;
+    for (int i = 0; i < 3; ++i) {
+        const int fields[3] = {(int)DF_COUNT, (int)CF_COUNT, (int)XF_COUNT};
+        const size_t words = (size_t)fields[i] * num_ranks;
         MC_HIP(hipMalloc((void**)&w->d_tbl[i], words * sizeof(uint64_t)));
     }
     MC_HIP(hipMalloc(&w->d_zero_row, kZeroRowBytes));
@@ -603,13 +606,14 @@ int mc_ep_world_destroy(mc_ep_world_t* w) {
     if (!w) return MC_EP_OK;
     DeviceGuard guard(w->device);
     (void)hipDeviceSynchronize();
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 3; ++i)
         if (w->d_tbl[i]) (void)hipFree(w->d_tbl[i]);
     if (w->d_routes) (void)hipFree(w->d_routes);
     if (w->d_ucount) (void)hipFree(w->d_ucount);
     if (w->d_ubegin) (void)hipFree(w->d_ubegin);
     if (w->d_selpos) (void)hipFree(w->d_selpos);
     if (w->d_ticket) (void)hipFree(w->d_ticket);
+    if (w->d_chunk_map) (void)hipFree(w->d_chunk_map);
     if (w->d_zero_row) (void)hipFree(w->d_zero_row);
     if (w->d_scale_stage) (void)hipFree(w->d_scale_stage);
     if (w->d_row_src) (void)hipFree(w->d_row_src);
@@ -679,6 +683,42 @@ int mc_ep_world_combine(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_t
     return world_combine_impl(w, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
                               active_ranks_ptrs, num_combined_tokens, hidden, num_topk, max_tokens, num_experts,
                               combined_x_ptrs, phases, (hipStream_t)stream_ptr);
+}
+
+int mc_ep_world_cast_back(mc_ep_world_t* w, const uint64_t* recv_x_ptrs, const uint64_t* recv_scales_ptrs,
+                          const uint64_t* recv_count_ptrs, uint64_t expert_factor_ptr, const uint64_t* out_ptrs,
+                          int hidden, int num_topk, int max_tokens, int num_experts, uint64_t stream_ptr) {
+    MC_ASSERT(w != nullptr);
+    const int R = w->R;
+    MC_ASSERT(num_experts > 0 && num_experts % R == 0);
+    MC_ASSERT(hidden > 0 && hidden % 128 == 0);
+    MC_ASSERT(max_tokens > 0 && num_topk >= 0);
+    MC_ASSERT(recv_x_ptrs != nullptr && recv_count_ptrs != nullptr && out_ptrs != nullptr);
+    const bool use_fp8 = recv_scales_ptrs != nullptr;
+    std::vector<uint64_t> tbl((size_t)XF_COUNT * R, 0);
+    for (int r = 0; r < R; ++r) {
+        if (recv_x_ptrs[r] != 0) {
+            MC_ASSERT(recv_count_ptrs[r] != 0 && out_ptrs[r] != 0);
+            MC_ASSERT(out_ptrs[r] != recv_x_ptrs[r] || !use_fp8);   // fp8 rows cannot be widened in place
+            if (use_fp8) MC_ASSERT(recv_scales_ptrs[r] != 0);
+        }
+        tbl[XF_RECV_X * R + r] = recv_x_ptrs[r];
+        tbl[XF_RECV_SCALES * R + r] = use_fp8 ? recv_scales_ptrs[r] : 0;
+        tbl[XF_RECV_COUNT * R + r] = recv_count_ptrs[r];
+        tbl[XF_OUT * R + r] = recv_x_ptrs[r] != 0 ? out_ptrs[r] : 0;
+    }
+    DeviceGuard guard(w->device);
+    hipStream_t stream = (hipStream_t)stream_ptr;
+    if (int rc = upload_table(w, 2, tbl, stream)) return rc;
+    Dims d{R, num_experts, num_topk, hidden, max_tokens, max_tokens};
+    // valid rows of the world: at most one per selection, and no more than the layout holds
+    long long max_rows = (long long)num_experts * R * max_tokens;
+    if (num_topk > 0 && (long long)R * max_tokens * num_topk < max_rows) max_rows = (long long)R * max_tokens * num_topk;
+    const size_t map_words = (size_t)(cast_back_chunks(max_rows, num_experts) + 1) * 4;
+    if (int rc = ensure_scratch(&w->d_chunk_map, &w->chunk_map_cap, map_words)) return rc;
+    MC_HIP(launch_cast_back(w->d_tbl[2], w->d_chunk_map, (const float*)expert_factor_ptr, use_fp8, max_rows, d,
+                            stream));
+    return MC_EP_OK;
 }
 
 int mc_ep_world_legacy_buffer_perf(mc_ep_world_t* w, const mc_ep_legacy_perf_tensors_t* t,

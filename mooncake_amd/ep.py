@@ -105,6 +105,17 @@ class World:
                              num_max_dispatch_tokens_per_rank, num_experts, combined_x_ptrs)(stream_ptr, phases)
 
 
+    def cast_back(self, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, expert_factor_ptr: int, out_ptrs,
+                  hidden: int, num_topk: int, num_max_dispatch_tokens_per_rank: int, num_experts: int,
+                  stream_ptr: int) -> None:
+        """Valid packed rows -> bf16 rows (fp8 payload times its scales; bf16 payload when
+        recv_scales_ptrs is None), times expert_factor[expert] when a factor array is given."""
+        u = _lib.u64_array
+        _lib.check(_lib.lib().mc_ep_world_cast_back(
+            self._h, u(recv_x_ptrs), u(recv_scales_ptrs) if recv_scales_ptrs is not None else None,
+            u(recv_count_ptrs), int(expert_factor_ptr), u(out_ptrs), hidden, num_topk,
+            num_max_dispatch_tokens_per_rank, num_experts, stream_ptr))
+
     def legacy_buffer_perf(self, tensors: Dict[str, Sequence[int]], num_tokens: int, hidden: int, num_topk: int,
                            num_local_experts: int, num_max_dispatch_tokens_per_rank: int, num_experts: int,
                            warmups: int = 20, iterations: int = 30, timeout_us: int = -1,

@@ -119,6 +119,22 @@ class WorldHarness:
         """Logical [R, L, R*max, H/128] view of the column-major scales."""
         return None if self.recv_scales_phys is None else self.recv_scales_phys.transpose(2, 3)
 
+    def cast_back(self, factor_per_expert: Optional[torch.Tensor] = None,
+                  stream: Optional[torch.cuda.Stream] = None, present: Optional[Sequence[int]] = None) -> None:
+        """expert_out = the dispatched rows as bf16 (times a per-expert factor), valid rows only, by the
+        library's consumer kernel."""
+        c = self.cfg
+        R = c.num_ranks
+        if self.expert_out is None:
+            self.alloc_combine_io()
+        self._factor = None if factor_per_expert is None else \
+            factor_per_expert.to(device=self.device, dtype=torch.float32).contiguous()
+        self.world.cast_back(self._ptrs(self.recv_x, R, present),
+                             self._ptrs(self.recv_scales_phys, R, present) if c.use_fp8 else None,
+                             self._ptrs(self.recv_count, R), 0 if self._factor is None else self._factor.data_ptr(),
+                             self._ptrs(self.expert_out, R), c.hidden, c.num_topk, c.max_tokens, c.num_experts,
+                             self._stream(stream))
+
     def fill_expert_out_from_recv(self, factor_per_expert: Optional[torch.Tensor] = None) -> None:
         """Mock expert: expert_out = dequantised dispatched rows (times a per-expert
         factor), rank by rank to bound temporaries."""

@@ -327,3 +327,35 @@ ORACLE_API uint64_t oracle_buffer_size_hint(int max_tokens, int hidden, int num_
     uint64_t data = (uint64_t)num_experts * (uint64_t)max_tokens * (2u * 16u + (uint64_t)hidden * 2u);
     return 4u * signaling + 4u * data;
 }
+
+/* The consumer of the packed layout.  per_token_cast_back
+ * (mooncake-wheel/tests/ep_test_utils.py:50-53) and dequantize_fp8
+ * (mooncake-ep/tests/test_ep_grid.py:43-48): f32(fp8) * scale per 128-element
+ * group, rounded to bf16; then, when factor != NULL, the grid test's mock
+ * expert (test_ep_grid.py:168-173): f32(that bf16) * factor[expert], rounded to
+ * bf16 again (a bf16 tensor times a scalar is computed in fp32 and rounded
+ * once).  recv_x is [E, RM, H] bytes (fp8) or bf16 when scales == NULL; scales
+ * is the physical column-major [E, H/128, RM]; only rows below count[e] are
+ * read or written. */
+ORACLE_API void oracle_cast_back(int E, int RM, int H, const void* recv_x, const float* scales,
+                                 const int32_t* count, const float* factor, uint16_t* out) {
+    const int G = H / 128;
+#pragma omp parallel for schedule(dynamic)
+    for (int e = 0; e < E; ++e) {
+        const int64_t rows = count[e] < 0 ? 0 : (count[e] > RM ? RM : count[e]);
+        for (int64_t row = 0; row < rows; ++row) {
+            const int64_t base = ((int64_t)e * RM + row) * H;
+            for (int j = 0; j < H; ++j) {
+                uint16_t v;
+                if (scales) {
+                    const float s = scales[((int64_t)e * G + j / 128) * RM + row];
+                    v = f32_to_bf16(e4m3fn_to_f32(((const uint8_t*)recv_x)[base + j]) * s);
+                } else {
+                    v = ((const uint16_t*)recv_x)[base + j];
+                }
+                if (factor) v = f32_to_bf16(bf16_to_f32(v) * factor[e]);
+                out[base + j] = v;
+            }
+        }
+    }
+}

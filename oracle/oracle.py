@@ -169,6 +169,26 @@ def combine(expert_out: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torc
     return out
 
 
+def cast_back(recv_x: torch.Tensor, scales: Optional[torch.Tensor], recv_count: torch.Tensor,
+              factor: Optional[torch.Tensor] = None, fill: int = 0) -> torch.Tensor:
+    """Valid packed rows -> bf16.  recv_x [R, L, RM, H] float8_e4m3fn / uint8 (with scales: the logical
+    [R, L, RM, H/128] view dispatch returns, or any tensor of that shape) or bf16 (scales None);
+    factor f32 [E] or None.  Rows at and beyond recv_count keep the 16-bit pattern `fill`."""
+    R, L, RM, H = recv_x.shape
+    phys = None
+    if scales is not None:
+        phys = scales.transpose(2, 3).contiguous().float()          # [R, L, H/128, RM]
+        raw = recv_x.contiguous().view(torch.uint8)
+    else:
+        assert recv_x.dtype == torch.bfloat16
+        raw = recv_x.contiguous()
+    out = torch.full((R, L, RM, H), fill, dtype=torch.int16)
+    cnt = recv_count.contiguous().to(torch.int32)
+    f = None if factor is None else factor.contiguous().float()
+    lib().oracle_cast_back(R * L, RM, H, _p(raw), _p(phys), _p(cnt), _p(f), _p(out))
+    return out.view(torch.bfloat16)
+
+
 def buffer_size_hint(max_tokens: int, hidden: int, num_ranks: int, num_experts: int) -> int:
     return int(lib().oracle_buffer_size_hint(max_tokens, hidden, num_ranks, num_experts))
 
