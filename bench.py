@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget for the cpu_baseline sample")
     ap.add_argument("--kernel-iters", type=int, default=30, help="timed launches per kernel for the roofline figures")
     ap.add_argument("--opt", action="append", default=[], help="library tuning option, name=value")
+    ap.add_argument("--graph", action="store_true",
+                    help="record the step into a HIP graph once and time replays instead of eager launches")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (the known-size "
                          "kernel that profiler FETCH_SIZE / WRITE_SIZE readings are scaled against)")
@@ -146,9 +148,19 @@ def main():
     h.cast_back()                          # expert outputs = dispatched rows cast back to bf16 (consumer kernel)
     torch.cuda.synchronize()
 
-    def step():
+    def eager_step():
         h.dispatch()
         h.combine()
+
+    step = eager_step
+    if args.graph:
+        # the step recorded once into a HIP graph and replayed (how serving loops run it)
+        eager_step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            eager_step()
+        step = graph.replay
 
     for _ in range(args.warmup):
         step()
@@ -200,7 +212,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": cfg.name, "num_ranks": cfg.num_ranks, "tokens_per_rank": cfg.tokens_per_rank,
                    "hidden": cfg.hidden, "num_experts": cfg.num_experts, "num_topk": cfg.num_topk,
-                   "use_fp8": cfg.use_fp8, "valid_selections": S, "seed": args.seed, "options": opts},
+                   "use_fp8": cfg.use_fp8, "valid_selections": S, "seed": args.seed, "options": opts,
+                   "launch": "graph replay" if args.graph else "eager"},
         "pct_of_hbm_peak": round(step_gbps / HBM_PEAK_GBPS * 100, 2),
         "dispatch_us": round(d_us, 2),
         "combine_us": round(c_us, 2),

@@ -83,6 +83,11 @@ struct mc_ep_world {
     hipStream_t comm_stream = nullptr;
     uint64_t* d_tbl[3] = {nullptr, nullptr, nullptr};   // dispatch, combine, consumer pointer tables
     std::vector<uint64_t> tbl_cache[3];                  // what the device tables hold
+    // Calls recorded into a HIP graph get tables of their own (a replay must not depend on what later
+    // eager calls leave in the shared ones); calls with equal tables share a slot.
+    uint64_t* d_captured_tbl[3] = {nullptr, nullptr, nullptr};
+    std::vector<std::vector<uint64_t>> captured_tbls[3];
+    bool dispatch_captured = false;                      // some dispatch of this world lives in a graph
     // routing state of the last dispatch (see RoutingScratch)
     int32_t* d_ucount = nullptr;
     size_t ucount_cap = 0;
@@ -105,6 +110,8 @@ struct mc_ep_world {
         int hidden = 0, num_topk = 0, max_tokens = 0, num_experts = 0;
         std::vector<uint64_t> topk_idx, recv_x, src_info, layout_range;
         std::vector<int32_t> num_tokens;
+        bool captured = false;                    // recorded into a graph, and which capture
+        unsigned long long capture_id = 0;
     } last;
     CombineRoute* d_routes = nullptr;             // combine's general path: one route per selection
     size_t route_cap = 0;                         // capacity in selections
@@ -151,8 +158,47 @@ struct DeviceGuard {
     }
 };
 
+// Tables a world keeps for calls recorded into graphs, per kind of call.
+constexpr int kCapturedTables = 256;
+
+struct Capture {
+    bool active = false;
+    unsigned long long id = 0;
+};
+
+// Whether work issued to `stream` is being recorded into a graph rather than run.
+int capture_of(hipStream_t stream, Capture* out) {
+    *out = Capture{};
+    if (stream == nullptr) return MC_EP_OK;   // the null stream cannot be captured
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long id = 0;
+    MC_HIP(hipStreamGetCaptureInfo(stream, &status, &id));
+    MC_ASSERT(status != hipStreamCaptureStatusInvalidated);
+    out->active = status == hipStreamCaptureStatusActive;
+    out->id = id;
+    return MC_EP_OK;
+}
+
+// Set while a call is being recorded: scratch cannot be allocated then.
+thread_local bool t_recording = false;
+
+struct RecordingScope {
+    bool prev;
+    explicit RecordingScope(bool on) : prev(t_recording) { t_recording = on; }
+    ~RecordingScope() { t_recording = prev; }
+};
+
+#define MC_NO_GROWTH_WHILE_RECORDING()                                                                         \
+    do {                                                                                                       \
+        if (t_recording)                                                                                       \
+            return fail(MC_EP_ERR_ASSERT,                                                                      \
+                        "Failed: the library's scratch memory would have to grow during stream capture; make "  \
+                        "the same call once outside the capture first");                                        \
+    } while (0)
+
 int ensure_routes(mc_ep_world* w, size_t selections) {
     if (selections <= w->route_cap) return MC_EP_OK;
+    MC_NO_GROWTH_WHILE_RECORDING();
     // grows only; the old table may still be read by queued kernels
     MC_HIP(hipDeviceSynchronize());
     if (w->d_routes) MC_HIP(hipFree(w->d_routes));
@@ -170,6 +216,7 @@ int ensure_routes(mc_ep_world* w, size_t selections) {
 template <typename T>
 int ensure_scratch(T** ptr, size_t* cap, size_t count) {
     if (count <= *cap) return MC_EP_OK;
+    MC_NO_GROWTH_WHILE_RECORDING();
     MC_HIP(hipDeviceSynchronize());
     if (*ptr) MC_HIP(hipFree(*ptr));
     *ptr = nullptr;
@@ -183,6 +230,7 @@ int ensure_scratch(T** ptr, size_t* cap, size_t count) {
 
 int ensure_scale_stage(mc_ep_world* w, size_t floats) {
     if (floats <= w->scale_stage_cap) return MC_EP_OK;
+    MC_NO_GROWTH_WHILE_RECORDING();
     MC_HIP(hipDeviceSynchronize());
     if (w->d_scale_stage) MC_HIP(hipFree(w->d_scale_stage));
     w->d_scale_stage = nullptr;
@@ -193,10 +241,38 @@ int ensure_scale_stage(mc_ep_world* w, size_t floats) {
     return MC_EP_OK;
 }
 
-int upload_table(mc_ep_world* w, int which, const std::vector<uint64_t>& tbl, hipStream_t stream) {
-    if (w->tbl_cache[which] == tbl) return MC_EP_OK;
-    MC_HIP(launch_table_write(w->d_tbl[which], tbl.data(), (int)tbl.size(), stream));
-    w->tbl_cache[which] = tbl;
+// Puts the call's rank table on the device and returns where.  Eager calls share one table per kind,
+// rewritten only when its contents change.  A call being recorded into a graph gets a slot that no
+// eager call touches and that is never rewritten; it is filled right away on the world's own
+// (non-capturing) stream, so the graph holds the call's kernels and nothing else.
+int upload_table(mc_ep_world* w, int which, const std::vector<uint64_t>& tbl, const Capture& cap,
+                 hipStream_t stream, const uint64_t** d_out) {
+    if (!cap.active) {
+        *d_out = w->d_tbl[which];
+        if (w->tbl_cache[which] == tbl) return MC_EP_OK;
+        MC_HIP(launch_table_write(w->d_tbl[which], tbl.data(), (int)tbl.size(), stream));
+        w->tbl_cache[which] = tbl;
+        return MC_EP_OK;
+    }
+    auto& known = w->captured_tbls[which];
+    size_t slot = 0;
+    while (slot < known.size() && known[slot] != tbl) ++slot;
+    if (slot == known.size()) {
+        if ((int)known.size() >= kCapturedTables)
+            return fail(MC_EP_ERR_ASSERT, "Failed: too many distinct calls of one world recorded into graphs (" +
+                                              std::to_string(kCapturedTables) + " sets of tensors per kind of call)");
+        uint64_t* d_new = w->d_captured_tbl[which] + slot * tbl.size();
+        MC_HIP(launch_table_write(d_new, tbl.data(), (int)tbl.size(), w->comm_stream));
+        // waiting for another stream is among the calls a capture in progress forbids by default; this
+        // one is safe (the world's stream takes no part in the capture), so say so for its duration
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        MC_HIP(hipThreadExchangeStreamCaptureMode(&mode));
+        const hipError_t waited = hipStreamSynchronize(w->comm_stream);
+        (void)hipThreadExchangeStreamCaptureMode(&mode);
+        MC_HIP(waited);
+        known.push_back(tbl);
+    }
+    *d_out = w->d_captured_tbl[which] + slot * tbl.size();
     return MC_EP_OK;
 }
 
@@ -267,6 +343,9 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         if (num_tokens[r] > tgrid) tgrid = num_tokens[r];
     }
     DeviceGuard guard(w->device);
+    Capture cap;
+    if (int rc = capture_of(stream, &cap)) return rc;
+    RecordingScope recording(cap.active);
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
     // the count kernel keeps per-wave counts and prefixes of every expert in LDS
     MC_ASSERT(count_lds_bytes(d) <= kMaxCountLdsBytes);
@@ -278,7 +357,8 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     if (int rc = ensure_scratch(&w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
     if (int rc = ensure_scratch(&w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
     if (int rc = ensure_scratch(&w->d_ticket, &w->ticket_cap, (size_t)1)) return rc;
-    if (int rc = upload_table(w, 0, tbl, stream)) return rc;
+    const uint64_t* d_tbl = nullptr;
+    if (int rc = upload_table(w, 0, tbl, cap, stream, &d_tbl)) return rc;
 
     const bool uni = w->tuning.uniform != 0;
     DispatchSource src;
@@ -287,7 +367,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     src.tokens = uniform_tokens(num_tokens, R, uni);
     const RoutingScratch sc = routing_scratch(w);
     if (phases & MC_EP_PHASE_LAYOUT) {
-        MC_HIP(launch_count(w->d_tbl[0], sc, src, d, stream));
+        MC_HIP(launch_count(d_tbl, sc, src, d, stream));
         auto& ld = w->last;
         ld.valid = true;
         ld.hidden = hidden; ld.num_topk = num_topk; ld.max_tokens = max_tokens; ld.num_experts = num_experts;
@@ -296,6 +376,9 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         ld.src_info.assign(src_info, src_info + R);
         ld.layout_range.assign(layout_range, layout_range + R);
         ld.num_tokens.assign(num_tokens, num_tokens + R);
+        ld.captured = cap.active;
+        ld.capture_id = cap.id;
+        if (cap.active) w->dispatch_captured = true;
     }
     if ((phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
         float* stage = nullptr;
@@ -303,7 +386,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
             if (int rc = ensure_scale_stage(w, (size_t)R * max_tokens * (hidden / 128))) return rc;
             stage = w->d_scale_stage;
         }
-        MC_HIP(launch_pack(w->d_tbl[0], sc, src, stage, d, use_fp8 != 0, w->tuning,
+        MC_HIP(launch_pack(d_tbl, sc, src, stage, d, use_fp8 != 0, w->tuning,
                            (phases & MC_EP_PHASE_DATA) != 0, (phases & MC_EP_PHASE_FINISH) != 0, stream));
     }
     return MC_EP_OK;
@@ -339,7 +422,11 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     }
     if (tgrid == 0) return MC_EP_OK;
     DeviceGuard guard(w->device);
-    if (int rc = upload_table(w, 1, tbl, stream)) return rc;
+    Capture cap;
+    if (int rc = capture_of(stream, &cap)) return rc;
+    RecordingScope recording(cap.active);
+    const uint64_t* d_tbl = nullptr;
+    if (int rc = upload_table(w, 1, tbl, cap, stream, &d_tbl)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
 
     // Is this the handle (and the routing input) of the last dispatch?  Then the
@@ -350,6 +437,10 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     const auto& ld = w->last;
     bool direct = w->tuning.combine_direct != 0 && ld.valid && ld.hidden == hidden && ld.num_topk == num_topk &&
                   ld.max_tokens == max_tokens && ld.num_experts == num_experts;
+    // "Last" is about the order on the device.  Graph replays run dispatches the host never sees, so: a
+    // recorded combine trusts only a dispatch recorded in the same capture, and once a dispatch of this
+    // world lives in a graph, eager combines resolve their handle (always right) instead.
+    direct = direct && (cap.active ? (ld.captured && ld.capture_id == cap.id) : !w->dispatch_captured);
     for (int r = 0; r < R && direct; ++r) {
         if (num_tokens[r] > 0) direct = topk_idx[r] == ld.topk_idx[r] && num_tokens[r] == ld.num_tokens[r];
         if (direct && x[r] != 0)
@@ -362,15 +453,21 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     src.topk_weights = uniform_ptr(topk_weights, R, uni);
     src.out = uniform_ptr(out, R, uni);
     src.tokens = uniform_tokens(num_tokens, R, uni);
+    // sized on every path, so that an eager call prepares the world for any recorded one of the same shape
+    if (int rc = ensure_routes(w, (size_t)R * max_tokens * num_topk)) return rc;
     if (!direct) {
-        if (int rc = ensure_routes(w, (size_t)R * max_tokens * num_topk)) return rc;
         if (phases & MC_EP_PHASE_LAYOUT) {
             w->stamp += 1;
-            MC_HIP(launch_resolve(w->d_tbl[1], w->d_routes, w->stamp, d, w->tuning, stream));
+            // every replay of a recorded call carries the same stamp: clear the routes so that none of an
+            // earlier replay passes for this one's
+            if (cap.active)
+                MC_HIP(launch_fill_u32(w->d_routes, 0u, (size_t)R * max_tokens * num_topk * (sizeof(CombineRoute) / 4),
+                                       stream));
+            MC_HIP(launch_resolve(d_tbl, w->d_routes, w->stamp, d, w->tuning, stream));
         }
     }
     if (phases & MC_EP_PHASE_DATA)
-        MC_HIP(launch_reduce(w->d_tbl[1], w->d_routes, w->stamp, routing_scratch(w), direct, src, w->d_zero_row, d,
+        MC_HIP(launch_reduce(d_tbl, w->d_routes, w->stamp, routing_scratch(w), direct, src, w->d_zero_row, d,
                              w->tuning, stream));
     return MC_EP_OK;
 }
@@ -562,6 +659,18 @@ std::string missing_ranks_message(const char* what) {
            " is a collective over the world's live ranks and not every one of them has called it yet";
 }
 
+// The per-rank calls form a round out of several host calls, with events between streams: that
+// bookkeeping is not something a graph can hold.  Whole-world calls can be recorded.
+int refuse_capture(uint64_t stream_ptr) {
+    Capture cap;
+    if (int rc = capture_of((hipStream_t)stream_ptr, &cap)) return rc;
+    if (cap.active)
+        return fail(MC_EP_ERR_UNSUPPORTED,
+                    "Failed: per-rank Buffer calls cannot be recorded into a graph; record mc_ep_world_dispatch / "
+                    "mc_ep_world_combine instead");
+    return MC_EP_OK;
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -592,6 +701,7 @@ int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
         const int fields[3] = {(int)DF_COUNT, (int)CF_COUNT, (int)XF_COUNT};
         const size_t words = (size_t)fields[i] * num_ranks;
         MC_HIP(hipMalloc((void**)&w->d_tbl[i], words * sizeof(uint64_t)));
+        MC_HIP(hipMalloc((void**)&w->d_captured_tbl[i], (size_t)kCapturedTables * words * sizeof(uint64_t)));
     }
     MC_HIP(hipMalloc(&w->d_zero_row, kZeroRowBytes));
     MC_HIP(hipMemset(w->d_zero_row, 0, kZeroRowBytes));
@@ -606,8 +716,10 @@ int mc_ep_world_destroy(mc_ep_world_t* w) {
     if (!w) return MC_EP_OK;
     DeviceGuard guard(w->device);
     (void)hipDeviceSynchronize();
-    for (int i = 0; i < 3; ++i)
+    for (int i = 0; i < 3; ++i) {
         if (w->d_tbl[i]) (void)hipFree(w->d_tbl[i]);
+        if (w->d_captured_tbl[i]) (void)hipFree(w->d_captured_tbl[i]);
+    }
     if (w->d_routes) (void)hipFree(w->d_routes);
     if (w->d_ucount) (void)hipFree(w->d_ucount);
     if (w->d_ubegin) (void)hipFree(w->d_ubegin);
@@ -709,14 +821,18 @@ int mc_ep_world_cast_back(mc_ep_world_t* w, const uint64_t* recv_x_ptrs, const u
     }
     DeviceGuard guard(w->device);
     hipStream_t stream = (hipStream_t)stream_ptr;
-    if (int rc = upload_table(w, 2, tbl, stream)) return rc;
+    Capture cap;
+    if (int rc = capture_of(stream, &cap)) return rc;
+    RecordingScope recording(cap.active);
+    const uint64_t* d_tbl = nullptr;
+    if (int rc = upload_table(w, 2, tbl, cap, stream, &d_tbl)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, max_tokens};
     // valid rows of the world: at most one per selection, and no more than the layout holds
     long long max_rows = (long long)num_experts * R * max_tokens;
     if (num_topk > 0 && (long long)R * max_tokens * num_topk < max_rows) max_rows = (long long)R * max_tokens * num_topk;
     const size_t map_words = (size_t)(cast_back_chunks(max_rows, num_experts) + 1) * 4;
     if (int rc = ensure_scratch(&w->d_chunk_map, &w->chunk_map_cap, map_words)) return rc;
-    MC_HIP(launch_cast_back(w->d_tbl[2], w->d_chunk_map, (const float*)expert_factor_ptr, use_fp8, max_rows, d,
+    MC_HIP(launch_cast_back(d_tbl, w->d_chunk_map, (const float*)expert_factor_ptr, use_fp8, max_rows, d,
                             stream));
     return MC_EP_OK;
 }
@@ -839,6 +955,7 @@ int mc_ep_buffer_dispatch(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_p
     MC_ASSERT(b != nullptr && event_out != nullptr && hook_out != nullptr);
     *event_out = nullptr;
     *hook_out = nullptr;
+    if (int rc = refuse_capture(compute_stream_ptr)) return rc;
     mc_ep_world* w = b->world;
     const int num_ranks = w->R;
     // mooncake_ep_buffer.cpp:202-206
@@ -898,6 +1015,7 @@ int mc_ep_buffer_combine(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_pt
     MC_ASSERT(b != nullptr && event_out != nullptr && hook_out != nullptr);
     *event_out = nullptr;
     *hook_out = nullptr;
+    if (int rc = refuse_capture(compute_stream_ptr)) return rc;
     mc_ep_world* w = b->world;
     const int num_ranks = w->R;
     if (zero_copy)
