@@ -867,7 +867,6 @@ __global__ __launch_bounds__(256) void cast_back_kernel(const uint64_t* __restri
     // of its two 16-byte stores lands in a run of 1 KB written by the wave as a whole.
     // Piece p covers columns col0 + p * 512 + lane * 8 .. + 7; 16 lanes share a scale group.
     constexpr int kHalf = kCastCols / 2;
-    constexpr int kIn = FP8 ? 8 : 16;               // payload bytes per piece
     bool on[2];
     int64_t in_off[2], out_off[2];
     const float* scale_col[2];

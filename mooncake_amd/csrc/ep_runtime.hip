@@ -46,6 +46,7 @@ int fail(int code, const std::string& msg) {
 // One collective call (a "round"): the j-th dispatch (or combine) of every live rank.
 struct Round {
     bool launched = false;
+    std::string failure;          // why the round's launch failed, if it did
     hipEvent_t done = nullptr;
     ~Round() {
         if (done) (void)hipEventDestroy(done);
@@ -126,6 +127,23 @@ struct mc_ep_world {
     std::deque<PendingRound<CombinePost>> combine_rounds;
     std::vector<long long> dispatch_calls, combine_calls;   // calls made per rank
     long long dispatch_base = 0, combine_base = 0;          // index of the front round
+
+    mc_ep_world() = default;
+    mc_ep_world(const mc_ep_world&) = delete;
+    mc_ep_world& operator=(const mc_ep_world&) = delete;
+    // also runs when creation fails half way
+    ~mc_ep_world() {
+        int prev = -1;
+        const bool switched = hipGetDevice(&prev) == hipSuccess && prev != device && hipSetDevice(device) == hipSuccess;
+        (void)hipDeviceSynchronize();
+        void* owned[] = {d_tbl[0], d_tbl[1], d_tbl[2], d_captured_tbl[0], d_captured_tbl[1], d_captured_tbl[2],
+                         d_ucount, d_ubegin, d_selpos, d_row_src, d_counts, d_ticket, d_chunk_map, d_routes,
+                         d_scale_stage, d_zero_row};
+        for (void* p : owned)
+            if (p) (void)hipFree(p);
+        if (comm_stream) (void)hipStreamDestroy(comm_stream);
+        if (switched) (void)hipSetDevice(prev);
+    }
 };
 
 struct mc_ep_buffer {
@@ -625,6 +643,7 @@ bool round_complete(const mc_ep_world* w, const PendingRound<Post>& pr) {
 int drain_dispatch(mc_ep_world* w) {
     while (!w->dispatch_rounds.empty() && round_complete(w, w->dispatch_rounds.front())) {
         int e = launch_dispatch_round(w, w->dispatch_rounds.front());
+        if (e) w->dispatch_rounds.front().state->failure = g_last_error;
         w->dispatch_rounds.pop_front();
         w->dispatch_base++;
         if (e) return e;
@@ -635,6 +654,7 @@ int drain_dispatch(mc_ep_world* w) {
 int drain_combine(mc_ep_world* w) {
     while (!w->combine_rounds.empty() && round_complete(w, w->combine_rounds.front())) {
         int e = launch_combine_round(w, w->combine_rounds.front());
+        if (e) w->combine_rounds.front().state->failure = g_last_error;
         w->combine_rounds.pop_front();
         w->combine_base++;
         if (e) return e;
@@ -654,9 +674,14 @@ PendingRound<Post>& round_for_call(mc_ep_world* w, std::deque<PendingRound<Post>
     return rounds[(size_t)(call_index - base)];
 }
 
-std::string missing_ranks_message(const char* what) {
-    return std::string("Failed: ") + what +
-           " is a collective over the world's live ranks and not every one of them has called it yet";
+// What a waiter on a round that cannot complete is told: either the launch failed (the call that
+// completed the round got the error; the other ranks learn it here), or ranks are still missing.
+int round_not_ready(const Round* round) {
+    if (round != nullptr && !round->failure.empty())
+        return fail(MC_EP_ERR_ASSERT, "Failed: the collective could not be launched: " + round->failure);
+    return fail(MC_EP_ERR_PENDING,
+                "Failed: the call is a collective over the world's live ranks and not every one of them has "
+                "called it yet");
 }
 
 // The per-rank calls form a round out of several host calls, with events between streams: that
@@ -713,25 +738,7 @@ int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
 }
 
 int mc_ep_world_destroy(mc_ep_world_t* w) {
-    if (!w) return MC_EP_OK;
-    DeviceGuard guard(w->device);
-    (void)hipDeviceSynchronize();
-    for (int i = 0; i < 3; ++i) {
-        if (w->d_tbl[i]) (void)hipFree(w->d_tbl[i]);
-        if (w->d_captured_tbl[i]) (void)hipFree(w->d_captured_tbl[i]);
-    }
-    if (w->d_routes) (void)hipFree(w->d_routes);
-    if (w->d_ucount) (void)hipFree(w->d_ucount);
-    if (w->d_ubegin) (void)hipFree(w->d_ubegin);
-    if (w->d_selpos) (void)hipFree(w->d_selpos);
-    if (w->d_ticket) (void)hipFree(w->d_ticket);
-    if (w->d_chunk_map) (void)hipFree(w->d_chunk_map);
-    if (w->d_zero_row) (void)hipFree(w->d_zero_row);
-    if (w->d_scale_stage) (void)hipFree(w->d_scale_stage);
-    if (w->d_row_src) (void)hipFree(w->d_row_src);
-    if (w->d_counts) (void)hipFree(w->d_counts);
-    if (w->comm_stream) (void)hipStreamDestroy(w->comm_stream);
-    delete w;
+    delete w;   // ~mc_ep_world waits for the device and releases what the world owns
     return MC_EP_OK;
 }
 
@@ -1079,7 +1086,7 @@ int mc_ep_event_current_stream_wait(mc_ep_event_t* ev, uint64_t stream_ptr) {
         MC_HIP(hipStreamWaitEvent((hipStream_t)stream_ptr, ev->own, 0));
         return MC_EP_OK;
     }
-    if (!ev->round || !ev->round->launched) return fail(MC_EP_ERR_PENDING, missing_ranks_message("the call"));
+    if (!ev->round || !ev->round->launched) return round_not_ready(ev->round.get());
     MC_HIP(hipStreamWaitEvent((hipStream_t)stream_ptr, ev->round->done, 0));
     return MC_EP_OK;
 }
@@ -1090,7 +1097,7 @@ int mc_ep_event_synchronize(mc_ep_event_t* ev) {
         MC_HIP(hipEventSynchronize(ev->own));
         return MC_EP_OK;
     }
-    if (!ev->round || !ev->round->launched) return fail(MC_EP_ERR_PENDING, missing_ranks_message("the call"));
+    if (!ev->round || !ev->round->launched) return round_not_ready(ev->round.get());
     MC_HIP(hipEventSynchronize(ev->round->done));
     return MC_EP_OK;
 }
@@ -1104,7 +1111,7 @@ int mc_ep_event_destroy(mc_ep_event_t* ev) {
 
 int mc_ep_hook_call(mc_ep_hook_t* h) {
     MC_ASSERT(h != nullptr);
-    if (!h->round || !h->round->launched) return fail(MC_EP_ERR_PENDING, missing_ranks_message("the call"));
+    if (!h->round || !h->round->launched) return round_not_ready(h->round.get());
     MC_HIP(hipStreamWaitEvent(h->stream, h->round->done, 0));
     return MC_EP_OK;
 }

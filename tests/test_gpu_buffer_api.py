@@ -239,6 +239,26 @@ def test_collective_rounds_and_pending_errors(gpu_device):
     assert not torch.equal(ra0[0][:, :4], rb0[0][:, :4])
 
 
+def test_a_round_that_cannot_launch_tells_every_waiter(gpu_device):
+    """Ranks that disagree about the shape of a collective: the call that completes the round fails, and the
+    rank that was already waiting on it learns why instead of seeing a round that is pending for ever."""
+    announce("failed round")
+    world, bufs = make_world(2, 16, 256, 4)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(16, 256, generator=g).to(torch.bfloat16).cuda()
+    idx = torch.topk(torch.randn(16, 4, generator=g), 2, dim=-1)[1].cuda()
+    first = bufs[0].dispatch(x, idx, None, 16, 4, -1, use_fp8=False, async_finish=True)
+    with pytest.raises(RuntimeError, match="Failed: Assertion"):
+        bufs[1].dispatch(x, idx[:, :1].contiguous(), None, 16, 4, -1, use_fp8=False)       # top-1 against top-2
+    with pytest.raises(RuntimeError, match="could not be launched"):
+        first[3].current_stream_wait()
+    # the world goes on with the next round
+    a = bufs[0].dispatch(x, idx, None, 16, 4, -1, use_fp8=False)
+    b = bufs[1].dispatch(x, idx, None, 16, 4, -1, use_fp8=False)
+    torch.cuda.synchronize()
+    assert int(a[1].sum() + b[1].sum()) == 2 * 16 * 2
+
+
 def test_host_assertions_and_unsupported(gpu_device):
     announce("host assertions")
     world, groups = LogicalGroup.make_world(2)
