@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget for the cpu_baseline sample")
     ap.add_argument("--kernel-iters", type=int, default=30, help="timed launches per kernel for the roofline figures")
     ap.add_argument("--opt", action="append", default=[], help="library tuning option, name=value")
+    ap.add_argument("--flush-mb", type=int, default=0,
+                    help="write this many MiB before every step of the per-kernel timing loop (cache flush)")
     ap.add_argument("--graph", action="store_true",
                     help="record the step into a HIP graph once and time replays instead of eager launches")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
@@ -51,7 +53,7 @@ def parse_args():
     return ap.parse_args()
 
 
-def time_pipeline(h, lib, iters):
+def time_pipeline(h, lib, iters, flush=None):
     """Device time of each kernel inside the running dispatch -> combine
     pipeline: events on the launch stream between the phases of every step, no
     host synchronisation inside the loop, so each kernel starts on the cache
@@ -66,6 +68,8 @@ def time_pipeline(h, lib, iters):
     marks = []
     for _ in range(iters + 2):
         ev = [torch.cuda.Event(enable_timing=True) for _ in range(len(phases) + 1)]
+        if flush is not None:
+            flush.zero_()       # the reference's cache flush between iterations (ep_test_utils.py:79-104), untimed
         ev[0].record()
         for i, (_, fn, ph) in enumerate(phases):
             fn(phases=ph)
@@ -174,7 +178,8 @@ def main():
     step_gbps = (alg["dispatch"] + alg["combine"]) / (elapsed / args.steps) / 1e9
 
     # per-kernel device times, measured live inside the pipeline
-    t = time_pipeline(h, _lib, args.kernel_iters)
+    flush = torch.empty(args.flush_mb << 20, dtype=torch.uint8, device="cuda:0") if args.flush_mb > 0 else None
+    t = time_pipeline(h, _lib, args.kernel_iters, flush)
     d_us = sum(t[k][0] for k in ("layout", "pack", "scales") if k in t)
     c_us = sum(t[k][0] for k in ("resolve", "reduce"))
     pack_us, red_us = t["pack"][0], t["reduce"][0]
