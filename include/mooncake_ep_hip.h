@@ -73,7 +73,7 @@ int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
 /* Tuning knobs for measurement sweeps ("pack_variant", "pack_waves",
  * "combine_chunks", "combine_waves", "combine_nt", "combine_direct", "uniform",
  * "pack_nt",
- * "scale_mode"). */
+ * "scale_mode", "routing_sum"). */
 int mc_ep_world_set_option(mc_ep_world_t* world, const char* name, int value);
 int mc_ep_world_get_option(const mc_ep_world_t* world, const char* name, int* value);
 

@@ -61,9 +61,24 @@ struct TableChunk {
 //     row(sel) = ubegin[unit(sel)][expert(sel)] + selpos[sel]
 // which is the deterministic order source rank ascending, token ascending.
 constexpr int kUnitSelections = 256;
+// With units of 1024 selections and few enough of them, the data kernels add up the counts of the
+// earlier units themselves and the prefix pass rides along in the pack launch: one launch less.
+constexpr int kBigUnitSelections = 1024;
+constexpr int kMaxSummedUnits = 64;
+
+// How the world's selections are cut into units and how packed rows come out of the unit counts.
+struct UnitPlan {
+    int per_rank = 0;   // units per rank
+    int shift = 8;      // log2(selections per unit)
+    int total = 0;      // R * per_rank
+    int summed = 0;     // 1: the data kernels of dispatch sum earlier units' counts themselves
+    int carried = 0;    // 1: the prefix pass rides in the pack launch (needs summed)
+    int selections() const { return 1 << shift; }
+};
 
 struct RoutingScratch {
     int32_t* ucount;     // [U, E]  selections of unit u that name expert e
+    int32_t* ucount_t;   // [E, kMaxSummedUnits]  the same, expert-major (summed plan only)
     int32_t* ubegin;     // [U, E]  exclusive prefix of ucount over units
     int32_t* selpos;     // [R * max_tokens * K]  position inside (unit, expert); -1: no valid expert
     int32_t* counts;     // [E]     rows per expert (0 for experts of ranks that take no part)
@@ -105,8 +120,9 @@ struct Dims {
     int H;            // hidden
     int max_tokens;   // num_max_dispatch_tokens_per_rank
     int Tgrid;        // max over ranks of T_r (grid extent in tokens per rank)
-    int units_per_rank() const { return (int)(((long long)max_tokens * K + kUnitSelections - 1) / kUnitSelections); }
-    int units() const { return R * units_per_rank(); }
+    UnitPlan plan;    // set by plan_units()
+    int units_per_rank() const { return plan.per_rank; }
+    int units() const { return plan.total; }
 };
 
 // Tuning knobs, settable at run time for measurement sweeps.
@@ -120,7 +136,11 @@ struct Tuning {
     int combine_chunks = 0;    // 16-byte chunks per lane in the combine kernel (1 or 2); 0: by top-k
     int combine_waves = 4;     // waves per block in the combine kernel
     int combine_nt = 3;        // bit 0: streaming loads, bit 1: streaming stores
+    int routing_sum = 1;       // allow the summed routing plan (see UnitPlan) where the shape permits
 };
+
+// Chooses the unit plan for a shape (summed when allowed, the shape permits and there are tokens).
+void plan_units(Dims& d, const Tuning& t);
 
 hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_words, hipStream_t stream);
 

@@ -115,7 +115,7 @@ __device__ __forceinline__ uint64_t rank_ptr(const uint64_t* __restrict__ tbl, c
     return p.base != 0 ? p.base + (uint64_t)((int64_t)r * p.stride) : tbl[field * R + r];
 }
 
-// One block per unit (kUnitSelections consecutive (token, k) selections of one rank), one
+// One block per unit (UNIT consecutive (token, k) selections of one rank), one
 // selection per thread.  Each index is read exactly once.
 //   1. inside a wave, selections naming the same expert are ranked by lane
 //      (a 64-bit lane mask per expert in LDS, filled by LDS atomics);
@@ -126,11 +126,12 @@ __device__ __forceinline__ uint64_t rank_ptr(const uint64_t* __restrict__ tbl, c
 // (A token is expected to name an expert at most once; if it names one twice,
 // each occurrence gets its own row, as in the reference kernel, which sends
 // once per k: mooncake_ep_kernel.cu:230,273.)
-__global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* __restrict__ tbl, RoutingScratch sc,
-                                                                 DispatchSource src, int R, int E, int K,
-                                                                 int max_tokens, int upr) {
+template <int UNIT>
+__global__ __launch_bounds__(UNIT) void count_kernel(const uint64_t* __restrict__ tbl, RoutingScratch sc,
+                                                      DispatchSource src, int R, int E, int K, int max_tokens,
+                                                      int upr) {
     extern __shared__ unsigned long long lds_count[];
-    constexpr int NW = kUnitSelections / 64;
+    constexpr int NW = UNIT / 64;
     unsigned long long* wmask = lds_count;                     // [NW][E] lanes of the wave that name e
     uint16_t* wpre = (uint16_t*)(lds_count + (size_t)NW * E);  // [NW][E] selections of e in earlier waves
 
@@ -140,11 +141,11 @@ __global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int T = src.tokens >= 0 ? src.tokens : (int)tbl[DF_NUM_TOKENS * R + r];
     const int n = T * K;
-    const int sel = c * kUnitSelections + tid;                 // index into the rank's [T, K] list
+    const int sel = c * UNIT + tid;                            // index into the rank's [T, K] list
 
     int64_t e64 = -1;
     if (sel < n) e64 = ((const int64_t*)rank_ptr(tbl, src.topk_idx, DF_TOPK_IDX, R, r))[sel];
-    for (int i = tid; i < NW * E; i += kUnitSelections) wmask[i] = 0;
+    for (int i = tid; i < NW * E; i += UNIT) wmask[i] = 0;
     const bool valid = e64 >= 0 && e64 < (int64_t)E;
     const int e = valid ? (int)e64 : 0;
     __syncthreads();
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* 
     __syncthreads();
     const int rank_in_wave = valid ? __popcll(wmask[wave * E + e] & ((1ull << lane) - 1ull)) : 0;
 
-    for (int ee = tid; ee < E; ee += kUnitSelections) {
+    for (int ee = tid; ee < E; ee += UNIT) {
         int run = 0;
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
@@ -163,6 +164,8 @@ __global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* 
             run += __popcll(wmask[w * E + ee]);
         }
         sc.ucount[(int64_t)u * E + ee] = run;
+        // the summed plan (big units) also wants the counts expert-major, for the data kernels' sums
+        if (UNIT == kBigUnitSelections) sc.ucount_t[(int64_t)ee * kMaxSummedUnits + u] = run;
     }
     __syncthreads();
     if (sel < n) sc.selpos[(int64_t)r * max_tokens * K + sel] = valid ? (int)wpre[wave * E + e] + rank_in_wave : -1;
@@ -177,15 +180,10 @@ __global__ __launch_bounds__(kUnitSelections) void count_kernel(const uint64_t* 
 // XCD's whole L2, which costs more than a launch.)
 constexpr int kPrefixWaves = 4;
 
-__global__ __launch_bounds__(kPrefixWaves * 64) void prefix_kernel(const uint64_t* __restrict__ tbl,
-                                                                    RoutingScratch sc, int R, int E, int max_tokens,
-                                                                    int upr, int U) {
-    extern __shared__ int lds_prefix[];                     // [kPrefixWaves][U + 1]
+// The work of one wave for expert ee; pre is the wave's LDS row of U + 1 ints.
+__device__ __forceinline__ void prefix_expert(const uint64_t* __restrict__ tbl, const RoutingScratch& sc, int R, int E,
+                                              int max_tokens, int upr, int U, int ee, int* pre) {
     const int lane = wave_lane();
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int ee = blockIdx.x * kPrefixWaves + wave;
-    if (ee >= E) return;
-    int* pre = lds_prefix + (size_t)wave * (U + 1);
     int carry = 0;
     for (int u0 = 0; u0 < U; u0 += 64) {
         const int u = u0 + lane;
@@ -230,10 +228,21 @@ __global__ __launch_bounds__(kPrefixWaves * 64) void prefix_kernel(const uint64_
     }
 }
 
+__global__ __launch_bounds__(kPrefixWaves * 64) void prefix_kernel(const uint64_t* __restrict__ tbl,
+                                                                    RoutingScratch sc, int R, int E, int max_tokens,
+                                                                    int upr, int U) {
+    extern __shared__ int lds_prefix[];                     // [kPrefixWaves][U + 1]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ee = blockIdx.x * kPrefixWaves + wave;
+    if (ee >= E) return;
+    prefix_expert(tbl, sc, R, E, max_tokens, upr, U, ee, lds_prefix + (size_t)wave * (U + 1));
+}
+
 // The packed row of one (token, k) selection, from the routing state, in two
 // steps so that callers can put their own gathers next to the one dependent
 // load (ubegin) instead of behind it: every lane works on a valid selection
-// index (lanes >= K redo lane 0's), nothing is loaded under a branch.
+// index (slots >= K redo slot 0's), nothing is loaded under a branch.  `slot`
+// is which of the token's K selections the lane works on.
 struct SelKey {
     int e;          // global expert (0 when the selection is not valid)
     int q;          // rank that owns it
@@ -250,19 +259,20 @@ struct SelRow {
 };
 
 __device__ __forceinline__ SelKey selection_key(const int64_t* __restrict__ idx_row, const RoutingScratch& sc, int R,
-                                                int E, int K, int max_tokens, int upr, int r, int t, int lane) {
-    const int li = lane < K ? lane : 0;
+                                                int E, int K, int max_tokens, const UnitPlan& up, int r, int t,
+                                                int slot) {
+    const int li = slot < K ? slot : 0;
     const int i = t * K + li;
     const int64_t e64 = idx_row[li];
     const int pos = sc.selpos[(int64_t)r * max_tokens * K + i];
     SelKey k;
-    k.valid = lane < K && e64 >= 0 && e64 < (int64_t)E && pos >= 0;
+    k.valid = slot < K && e64 >= 0 && e64 < (int64_t)E && pos >= 0;
     k.e = k.valid ? (int)e64 : 0;
     const int L = E / R;
     k.q = k.e / L;
     k.le = k.e - k.q * L;
     k.pos = pos;
-    k.unit = r * upr + i / kUnitSelections;
+    k.unit = r * up.per_rank + (i >> up.shift);
     return k;
 }
 
@@ -275,9 +285,44 @@ __device__ __forceinline__ SelRow selection_row(const SelKey& k, int ubegin, int
     return s;
 }
 
+// Summed plan: the begin of (unit, expert) - the rows that earlier units give the expert - added up
+// on the fly from the unit counts.  The wave's lanes split into groups of sel_stride() lanes, one
+// group per selection of the token; a group's lanes take the earlier units four at a time and the
+// group sums up, so every lane of group k ends with selection k's begin.
+__device__ __forceinline__ int sel_stride(const UnitPlan& up, int K) {
+    if (!up.summed) return 1;                                  // table plan: lane k works on selection k
+    const int kp = K <= 1 ? 1 : (K <= 2 ? 2 : (K <= 4 ? 4 : (K <= 8 ? 8 : 16)));
+    return 64 / kp;
+}
+
+__device__ __forceinline__ int summed_begin(const RoutingScratch& sc, const SelKey& k, const UnitPlan& up, int r, int t,
+                                            int K, int j, int lps) {
+    const int unit_max = r * up.per_rank + ((t * K + K - 1) >> up.shift);   // wave-uniform bound
+    // a lane takes four consecutive units in one 16-byte load; rows of ucount_t are kMaxSummedUnits long
+    const int32_t* row = sc.ucount_t + (int64_t)k.e * kMaxSummedUnits;
+    int sum = 0;
+    for (int base = 0; base < unit_max; base += 4 * lps) {
+        const int u = base + 4 * j;
+        int4 v = make_int4(0, 0, 0, 0);
+        if (u < k.unit) v = *(const int4*)(row + u);
+        sum += (u < k.unit ? v.x : 0) + (u + 1 < k.unit ? v.y : 0) + (u + 2 < k.unit ? v.z : 0) +
+               (u + 3 < k.unit ? v.w : 0);
+    }
+    // sum over the group's lanes (4 to 64 of them): inside rows of 16 lanes in the DPP data path
+    sum += __builtin_amdgcn_mov_dpp(sum, 0xB1, 0xF, 0xF, true);                  // quad_perm [1,0,3,2]
+    sum += __builtin_amdgcn_mov_dpp(sum, 0x4E, 0xF, 0xF, true);                  // quad_perm [2,3,0,1]
+    if (lps >= 8) sum += __builtin_amdgcn_mov_dpp(sum, 0x141, 0xF, 0xF, true);   // row_half_mirror
+    if (lps >= 16) sum += __builtin_amdgcn_mov_dpp(sum, 0x140, 0xF, 0xF, true);  // row_mirror
+    if (lps >= 32) sum += __shfl_xor(sum, 16);
+    if (lps >= 64) sum += __shfl_xor(sum, 32);
+    return sum;
+}
+
 // ---------------------------------------------------------------------------
 // dispatch pack
 // ---------------------------------------------------------------------------
+constexpr int kMaxPackWaves = 8;     // waves per block the launcher may choose
+
 // One wave per (token, 1024-element slab).  Lanes 0..K-1 fetch the K resolved
 // destinations; the row slab is read once, quantised in registers and stored
 // K times.
@@ -286,27 +331,31 @@ struct PackDest {
     uint64_t scale;   // byte address of scales[le][0][slot] (fp8)
 };
 
-// Lanes 0..K-1 turn their selection into destination addresses.  The slab-0
-// wave of a token also records the row's source: src_info for the caller and
-// row_src for the scale transposition.
+// The lanes that work on selection k (lane k, or a group of sel_stride() lanes under the summed
+// plan) turn it into destination addresses; callers read them from lane k * sel_stride().  The
+// slab-0 wave of a token also records the row's source: src_info for the caller and row_src for the
+// scale transposition.
 template <bool FP8>
 __device__ __forceinline__ PackDest pack_destination(const uint64_t* __restrict__ tbl, const RoutingScratch& sc,
                                                      const int64_t* __restrict__ idx_row, int R, int E, int K,
-                                                     int max_tokens, int H, int upr, int r, int t, int slab,
-                                                     int lane) {
-    const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, upr, r, t, lane);
-    // the dependent gathers, side by side
-    const int ub = sc.ubegin[(int64_t)k.unit * E + k.e];
+                                                     int max_tokens, int H, const UnitPlan& up, int r, int t,
+                                                     int slab, int lane) {
+    const int stride = sel_stride(up, K);
+    const int slot = lane / stride, j = lane - slot * stride;
+    const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, up, r, t, slot);
+    // the dependent gathers, side by side; the table's come first because the summed begin waits for
+    // its own loads inside, and whatever is issued after that wait is a round trip later
     const uint64_t base = tbl[DF_RECV_X * R + k.q];
     const uint64_t sbase = FP8 ? tbl[DF_RECV_SCALES * R + k.q] : 0;
     const uint64_t info = (slab == 0) ? tbl[DF_SRC_INFO * R + k.q] : 0;
+    const int ub = up.summed ? summed_begin(sc, k, up, r, t, K, j, stride) : sc.ubegin[(int64_t)k.unit * E + k.e];
     const SelRow s = selection_row(k, ub, R, max_tokens);
     PackDest d = {0, 0};
     if (s.ok && base != 0) {
         const int64_t RM = (int64_t)R * max_tokens;
         d.row = base + (uint64_t)s.grow * (uint64_t)H * (FP8 ? 1 : 2);
         if (FP8) d.scale = sbase + (uint64_t)((int64_t)k.le * (H / 128) * RM + s.slot) * 4;
-        if (slab == 0) {
+        if (slab == 0 && j == 0) {
             ((int32_t*)info)[s.grow] = t;
             sc.row_src[(int64_t)k.e * RM + s.slot] = r * max_tokens + t;
         }
@@ -330,11 +379,21 @@ template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restrict__ tbl,
                                                         RoutingScratch sc, DispatchSource src,
                                                         float* __restrict__ scale_stage, int R, int E, int K,
-                                                        int max_tokens, int H, int upr, int slabs, int Tgrid,
+                                                        int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
                                                         int total_tasks) {
     const int lane = wave_lane();
-    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
+    if (up.carried) {
+        // the first E waves of the launch do the prefix pass (it needs the unit counts only)
+        __shared__ int lds_pre[kMaxPackWaves * (kMaxSummedUnits + 1)];
+        if (task < E) {
+            prefix_expert(tbl, sc, R, E, max_tokens, up.per_rank, up.total, task,
+                          lds_pre + (threadIdx.x >> 6) * (kMaxSummedUnits + 1));
+            return;
+        }
+        task -= E;
+    }
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
     const char* xtok;
@@ -349,7 +408,8 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
         a = load16<NTL>(xrow);
         b = load16<NTL>(xrow + 16);
     }
-    const PackDest dst = pack_destination<true>(tbl, sc, idx_row, R, E, K, max_tokens, H, upr, r, t, s, lane);
+    const PackDest dst = pack_destination<true>(tbl, sc, idx_row, R, E, K, max_tokens, H, up, r, t, s, lane);
+    const int sel_lanes = sel_stride(up, K);   // selection k's destination sits in lane k * sel_lanes
 
     float f[16];
     const uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
@@ -383,8 +443,8 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
     const bool scatter_scales = scale_lane && scale_stage == nullptr;
 
     for (int k = 0; k < K; ++k) {
-        const uint64_t row = read_lane_u64(dst.row, k);
-        const uint64_t sc = read_lane_u64(dst.scale, k);
+        const uint64_t row = read_lane_u64(dst.row, k * sel_lanes);
+        const uint64_t sc = read_lane_u64(dst.scale, k * sel_lanes);
         if (row == 0) continue;
         if (active) store16<NTS>((void*)(row + elem0), out);
         if (scatter_scales) *(float*)(sc + scale_off) = scale_inv;
@@ -398,11 +458,21 @@ template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __restrict__ tbl,
                                                               RoutingScratch sc, DispatchSource src,
                                                               float* __restrict__ scale_stage, int R, int E, int K,
-                                                              int max_tokens, int H, int upr, int slabs, int Tgrid,
+                                                              int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
                                                               int total_tasks) {
     const int lane = wave_lane();
-    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
+    if (up.carried) {
+        // the first E waves of the launch do the prefix pass (it needs the unit counts only)
+        __shared__ int lds_pre[kMaxPackWaves * (kMaxSummedUnits + 1)];
+        if (task < E) {
+            prefix_expert(tbl, sc, R, E, max_tokens, up.per_rank, up.total, task,
+                          lds_pre + (threadIdx.x >> 6) * (kMaxSummedUnits + 1));
+            return;
+        }
+        task -= E;
+    }
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
     const char* xbase;
@@ -419,7 +489,8 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
         v[p] = make_uint4(0, 0, 0, 0);
         if (active[p]) v[p] = load16<NTL>(xbase + (int64_t)elem[p] * 2);
     }
-    const PackDest dst = pack_destination<true>(tbl, sc, idx_row, R, E, K, max_tokens, H, upr, r, t, s, lane);
+    const PackDest dst = pack_destination<true>(tbl, sc, idx_row, R, E, K, max_tokens, H, up, r, t, s, lane);
+    const int sel_lanes = sel_stride(up, K);   // selection k's destination sits in lane k * sel_lanes
 
     uint2 out[2];
     float scale_inv[2];
@@ -454,8 +525,8 @@ __global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __r
     const bool scatter_scales = scale_lane && scale_stage == nullptr;
 
     for (int k = 0; k < K; ++k) {
-        const uint64_t row = read_lane_u64(dst.row, k);
-        const uint64_t sc = read_lane_u64(dst.scale, k);
+        const uint64_t row = read_lane_u64(dst.row, k * sel_lanes);
+        const uint64_t sc = read_lane_u64(dst.scale, k * sel_lanes);
         if (row == 0) continue;
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -472,11 +543,21 @@ template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restrict__ tbl,
                                                          RoutingScratch sc, DispatchSource src,
                                                          float* __restrict__ /*scale_stage*/, int R, int E, int K,
-                                                         int max_tokens, int H, int upr, int slabs, int Tgrid,
+                                                         int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
                                                          int total_tasks) {
     const int lane = wave_lane();
-    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
     if (task >= total_tasks) return;
+    if (up.carried) {
+        // the first E waves of the launch do the prefix pass (it needs the unit counts only)
+        __shared__ int lds_pre[kMaxPackWaves * (kMaxSummedUnits + 1)];
+        if (task < E) {
+            prefix_expert(tbl, sc, R, E, max_tokens, up.per_rank, up.total, task,
+                          lds_pre + (threadIdx.x >> 6) * (kMaxSummedUnits + 1));
+            return;
+        }
+        task -= E;
+    }
     const int n = task / slabs, s = task - n * slabs;
     const int r = n / Tgrid, t = n - r * Tgrid;
     const char* xbase;
@@ -494,10 +575,11 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
         v[p] = make_uint4(0, 0, 0, 0);
         if (active[p]) v[p] = load16<NTL>(xbase + off[p]);
     }
-    const PackDest dst = pack_destination<false>(tbl, sc, idx_row, R, E, K, max_tokens, H, upr, r, t, s, lane);
+    const PackDest dst = pack_destination<false>(tbl, sc, idx_row, R, E, K, max_tokens, H, up, r, t, s, lane);
+    const int sel_lanes = sel_stride(up, K);   // selection k's destination sits in lane k * sel_lanes
 
     for (int k = 0; k < K; ++k) {
-        const uint64_t row = read_lane_u64(dst.row, k);
+        const uint64_t row = read_lane_u64(dst.row, k * sel_lanes);
         if (row == 0) continue;
 #pragma unroll
         for (int p = 0; p < 2; ++p)
@@ -668,7 +750,7 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
                                                       const CombineRoute* __restrict__ routes, uint32_t stamp,
                                                       RoutingScratch sc, CombineSource cs,
                                                       const void* __restrict__ zero_row, int R, int E, int K,
-                                                      int max_tokens, int H, int upr, int slabs, int Tgrid,
+                                                      int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
                                                       int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
@@ -687,7 +769,7 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
         const float* w_row = (const float*)rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (int64_t)t * K;
         const float wl = w_row[lane < K ? lane : 0];
         const int32_t* active = (const int32_t*)tbl[CF_ACTIVE * R + r];
-        const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, upr, r, t, lane);
+        const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, up, r, t, lane);
         // the dependent gathers, side by side
         const int ub = sc.ubegin[(int64_t)k.unit * E + k.e];
         const uint64_t base = tbl[CF_X * R + k.q];
@@ -980,22 +1062,47 @@ hipError_t launch_clear_words(const uint64_t* h_ptrs, int n_ptrs, int words, hip
 }
 
 size_t count_lds_bytes(const Dims& d) {
-    return (size_t)(kUnitSelections / 64) * d.E * (8 + 2) + 64;
+    return (size_t)(d.plan.selections() / 64) * d.E * (8 + 2) + 64;
+}
+
+void plan_units(Dims& d, const Tuning& t) {
+    const long long per_rank_sel = (long long)d.max_tokens * d.K;
+    const long long big = (per_rank_sel + kBigUnitSelections - 1) / kBigUnitSelections;
+    const size_t big_lds = (size_t)(kBigUnitSelections / 64) * d.E * (8 + 2) + 64;
+    UnitPlan p;
+    if (t.routing_sum != 0 && d.Tgrid > 0 && big * d.R <= kMaxSummedUnits && big_lds <= kMaxCountLdsBytes) {
+        p.per_rank = (int)big;
+        p.shift = 10;
+        p.summed = 1;
+        p.carried = t.routing_sum == 1 ? 1 : 0;
+    } else {
+        p.per_rank = (int)((per_rank_sel + kUnitSelections - 1) / kUnitSelections);
+        p.shift = 8;
+        p.summed = 0;
+    }
+    p.total = d.R * p.per_rank;
+    d.plan = p;
 }
 
 hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, const Dims& d,
                         hipStream_t stream) {
     const size_t lds = count_lds_bytes(d);
     if (lds > kMaxCountLdsBytes) return hipErrorInvalidValue;
+    const void* kern = d.plan.shift == 10 ? (const void*)count_kernel<kBigUnitSelections>
+                                          : (const void*)count_kernel<kUnitSelections>;
     if (lds > 48 * 1024) {
-        hipError_t err =
-            hipFuncSetAttribute((const void*)count_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t err = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(count_kernel, dim3(d.units()), dim3(kUnitSelections), lds, stream, d_tbl, sc, src, d.R, d.E,
-                       d.K, d.max_tokens, d.units_per_rank());
+    if (d.plan.shift == 10)
+        hipLaunchKernelGGL(count_kernel<kBigUnitSelections>, dim3(d.units()), dim3(kBigUnitSelections), lds, stream,
+                           d_tbl, sc, src, d.R, d.E, d.K, d.max_tokens, d.units_per_rank());
+    else
+        hipLaunchKernelGGL(count_kernel<kUnitSelections>, dim3(d.units()), dim3(kUnitSelections), lds, stream, d_tbl,
+                           sc, src, d.R, d.E, d.K, d.max_tokens, d.units_per_rank());
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
+    if (d.plan.carried) return hipSuccess;   // the prefix pass rides in the pack launch
     const size_t plds = (size_t)kPrefixWaves * (d.units() + 1) * sizeof(int);
     if (plds > 60 * 1024) return hipErrorInvalidValue;
     hipLaunchKernelGGL(prefix_kernel, dim3((d.E + kPrefixWaves - 1) / kPrefixWaves), dim3(kPrefixWaves * 64), plds,
@@ -1003,19 +1110,20 @@ hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const D
     return hipGetLastError();
 }
 
-static int clamp_waves(int w) { return w < 1 ? 1 : (w > 8 ? 8 : w); }
+static int clamp_waves(int w) { return w < 1 ? 1 : (w > kMaxPackWaves ? kMaxPackWaves : w); }
 
 template <typename Kern>
 static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src,
                                 float* stage, const Dims& d, const Tuning& t, hipStream_t stream) {
     const int slabs = (d.H + 1023) / 1024;
-    const long long total = (long long)d.R * d.Tgrid * slabs;
+    long long total = (long long)d.R * d.Tgrid * slabs;
     if (total <= 0) return hipSuccess;
+    if (d.plan.carried) total += d.E;   // the prefix pass: a wave per expert in front of the data waves
     if (total > 0x7fffffffll) return hipErrorInvalidValue;
     const int wpb = clamp_waves(t.pack_waves);
     const int blocks = (int)((total + wpb - 1) / wpb);
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, sc, src, stage, d.R, d.E, d.K,
-                       d.max_tokens, d.H, d.units_per_rank(), slabs, d.Tgrid, (int)total);
+                       d.max_tokens, d.H, d.plan, slabs, d.Tgrid, (int)total);
     return hipGetLastError();
 }
 
@@ -1086,7 +1194,7 @@ static hipError_t launch_reduce_t(const ReduceLaunch& rl, const Dims& d, const T
 #define MCEP_REDUCE(A, B)                                                                                        \
     hipLaunchKernelGGL((reduce_kernel<KMAX, CH, A, B, DIRECT>), dim3(blocks), dim3(wpb * 64), 0, stream, rl.d_tbl, \
                        rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d.R, d.E, d.K, d.max_tokens, d.H,    \
-                       d.units_per_rank(), slabs, d.Tgrid, (int)total)
+                       d.plan, slabs, d.Tgrid, (int)total)
     if (ntl && nts) MCEP_REDUCE(true, true);
     else if (ntl) MCEP_REDUCE(true, false);
     else if (nts) MCEP_REDUCE(false, true);

@@ -94,6 +94,8 @@ struct mc_ep_world {
     size_t ucount_cap = 0;
     int32_t* d_ubegin = nullptr;
     size_t ubegin_cap = 0;
+    int32_t* d_ucount_t = nullptr;
+    size_t ucount_t_cap = 0;
     int32_t* d_selpos = nullptr;
     size_t selpos_cap = 0;
     int32_t* d_row_src = nullptr;
@@ -111,6 +113,7 @@ struct mc_ep_world {
         int hidden = 0, num_topk = 0, max_tokens = 0, num_experts = 0;
         std::vector<uint64_t> topk_idx, recv_x, src_info, layout_range;
         std::vector<int32_t> num_tokens;
+        UnitPlan plan;                            // how its routing state is laid out
         bool captured = false;                    // recorded into a graph, and which capture
         unsigned long long capture_id = 0;
     } last;
@@ -137,7 +140,7 @@ struct mc_ep_world {
         const bool switched = hipGetDevice(&prev) == hipSuccess && prev != device && hipSetDevice(device) == hipSuccess;
         (void)hipDeviceSynchronize();
         void* owned[] = {d_tbl[0], d_tbl[1], d_tbl[2], d_captured_tbl[0], d_captured_tbl[1], d_captured_tbl[2],
-                         d_ucount, d_ubegin, d_selpos, d_row_src, d_counts, d_ticket, d_chunk_map, d_routes,
+                         d_ucount, d_ucount_t, d_ubegin, d_selpos, d_row_src, d_counts, d_ticket, d_chunk_map, d_routes,
                          d_scale_stage, d_zero_row};
         for (void* p : owned)
             if (p) (void)hipFree(p);
@@ -326,7 +329,7 @@ int uniform_tokens(const int32_t* n, int R, bool enabled) {
 }
 
 RoutingScratch routing_scratch(const mc_ep_world* w) {
-    return RoutingScratch{w->d_ucount, w->d_ubegin, w->d_selpos, w->d_counts, w->d_row_src, w->d_ticket};
+    return RoutingScratch{w->d_ucount, w->d_ucount_t, w->d_ubegin, w->d_selpos, w->d_counts, w->d_row_src, w->d_ticket};
 }
 
 int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_idx, const int32_t* num_tokens,
@@ -365,12 +368,14 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     if (int rc = capture_of(stream, &cap)) return rc;
     RecordingScope recording(cap.active);
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
+    plan_units(d, w->tuning);
     // the count kernel keeps per-wave counts and prefixes of every expert in LDS
     MC_ASSERT(count_lds_bytes(d) <= kMaxCountLdsBytes);
     MC_ASSERT(d.units() <= kMaxUnits);
     const size_t UE = (size_t)d.units() * num_experts;
     if (int rc = ensure_scratch(&w->d_ucount, &w->ucount_cap, UE)) return rc;
     if (int rc = ensure_scratch(&w->d_ubegin, &w->ubegin_cap, UE)) return rc;
+    if (int rc = ensure_scratch(&w->d_ucount_t, &w->ucount_t_cap, (size_t)num_experts * kMaxSummedUnits)) return rc;
     if (int rc = ensure_scratch(&w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
     if (int rc = ensure_scratch(&w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
     if (int rc = ensure_scratch(&w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
@@ -394,6 +399,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         ld.src_info.assign(src_info, src_info + R);
         ld.layout_range.assign(layout_range, layout_range + R);
         ld.num_tokens.assign(num_tokens, num_tokens + R);
+        ld.plan = d.plan;
         ld.captured = cap.active;
         ld.capture_id = cap.id;
         if (cap.active) w->dispatch_captured = true;
@@ -446,6 +452,7 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     const uint64_t* d_tbl = nullptr;
     if (int rc = upload_table(w, 1, tbl, cap, stream, &d_tbl)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
+    d.plan = w->last.plan;   // read only when the last dispatch's routing state is reused
 
     // Is this the handle (and the routing input) of the last dispatch?  Then the
     // packed row of every selection is already known on the device.  Like the
@@ -760,6 +767,7 @@ static int* option_slot(Tuning& t, const char* name) {
     if (!strcmp(name, "scale_mode")) return &t.scale_mode;
     if (!strcmp(name, "combine_direct")) return &t.combine_direct;
     if (!strcmp(name, "combine_chunks")) return &t.combine_chunks;
+    if (!strcmp(name, "routing_sum")) return &t.routing_sum;
     if (!strcmp(name, "combine_waves")) return &t.combine_waves;
     if (!strcmp(name, "combine_nt")) return &t.combine_nt;
     return nullptr;

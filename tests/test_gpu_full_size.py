@@ -17,14 +17,15 @@ from tests.gpu_util import announce, compare_dispatch
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("name", CONFIG_ORDER)
-def test_named_config_full_size(gpu_device, oracle, name):
+@pytest.mark.parametrize("name,summed", [(n, 1) for n in CONFIG_ORDER] + [("dsv3_decode", 0), ("mixtral", 0)])
+def test_named_config_full_size(gpu_device, oracle, name, summed):
     cfg = CONFIGS[name]
-    announce(f"full size {cfg}")
+    announce(f"full size {cfg} routing_sum={summed}")
     data = generate(cfg, seed=0)
     R, T, E, K, L = cfg.num_ranks, cfg.tokens_per_rank, cfg.num_experts, cfg.num_topk, cfg.num_local_experts
     RM = R * cfg.max_tokens
     h = WorldHarness(cfg)
+    h.world.set_option("routing_sum", summed)
     h.load(data)
     h.alloc_dispatch_outputs(poison=False)
     # sentinel in the row right after each block's expected end, to see that padding is not touched

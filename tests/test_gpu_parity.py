@@ -57,7 +57,8 @@ def test_fp8_pack_variants_match_oracle(gpu_device, oracle, variant, nt, scale_m
     compare_dispatch(h, ref, check_poison=True)
 
 
-@pytest.mark.parametrize("opts", [{"uniform": 0}, {"pack_waves": 1}, {"pack_waves": 8}, {"pack_nt": 1}, {"pack_nt": 2}],
+@pytest.mark.parametrize("opts", [{"uniform": 0}, {"pack_waves": 1}, {"pack_waves": 8}, {"pack_nt": 1}, {"pack_nt": 2},
+                                  {"routing_sum": 0}, {"routing_sum": 0, "uniform": 0}],
                          ids=lambda o: "-".join(f"{k}{v}" for k, v in o.items()))
 def test_dispatch_tuning_options_match_oracle(gpu_device, oracle, opts):
     cfg = EPConfig("opts", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05)

@@ -36,16 +36,18 @@ def _case(seed: int):
     for _ in range(rng.randint(0, 2)):
         active[rng.randrange(R), rng.randrange(R)] = 0
     direct = rng.choice([0, 1])
-    return cfg, num_tokens, present, active, direct
+    summed = rng.choice([0, 1])      # both routing plans (prefix pass as its own launch, or inside pack)
+    return cfg, num_tokens, present, active, direct, summed
 
 
 @pytest.mark.parametrize("seed", range(32))
 def test_random_world(gpu_device, oracle, seed):
-    cfg, num_tokens, present, active, direct = _case(seed)
-    announce(f"random world seed={seed} {cfg} tokens={num_tokens} present={present} direct={direct}")
+    cfg, num_tokens, present, active, direct, summed = _case(seed)
+    announce(f"random world seed={seed} {cfg} tokens={num_tokens} present={present} direct={direct} summed={summed}")
     data = generate(cfg, seed=1000 + seed)
     h = WorldHarness(cfg, num_tokens=num_tokens)
     h.world.set_option("combine_direct", direct)
+    h.world.set_option("routing_sum", summed)
     h.load(data)
     h.alloc_dispatch_outputs(poison=True)
     h.alloc_combine_io()
