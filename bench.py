@@ -27,8 +27,8 @@ METRIC = "dispatch+combine µs & HBM GB/s (% peak), DSV3 decode 128 tok top-8 fp
 # the same counter reads for the library's plain copy kernel over 1 GiB
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Workloads not profiled report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("dsv3_decode", "reduce"): int((231869.9 * 2.0 + 57344.0 * 1.0) * 1024),
-    ("dsv3_decode", "pack"): int((30630.3 * 2.0 + 232294.0 * 1.0) * 1024),
+    ("dsv3_decode", "reduce"): int((231475.1 * 2.0 + 57344.0 * 1.0) * 1024),
+    ("dsv3_decode", "pack"): int((30769.1 * 2.0 + 232430.4 * 1.0) * 1024),
 }
 
 
