@@ -22,6 +22,11 @@ SMALL = [
     EPConfig("masked", 8, 64, 1024, 8, 2, False, masked_fraction=0.3),
     EPConfig("zipf_outliers", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05),
     shrink(CONFIGS["cpu_check"]),                                    # the contract's CPU-reference case, full size
+    # shapes at the edges of the routing plans: the count kernel's LDS beyond the default 48 KB (summed plan),
+    # too many experts for 1024-selection units' LDS, too many units to sum (both: table plan)
+    EPConfig("experts768", 8, 16, 256, 768, 8, True),
+    EPConfig("experts1024", 8, 16, 256, 1024, 8, False),
+    EPConfig("units80", 16, 600, 256, 32, 8, False),
 ]
 
 
