@@ -42,3 +42,27 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmooncake_ep_hip.so")
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.lib()
+
+
+def test_header_is_plain_c_and_structs_match_ctypes(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 on its own (no HIP, torch or C++ in it), and the
+    struct layouts the Python binding assumes are the ones a C compiler gives."""
+    import subprocess
+    from mooncake_amd import _lib
+    src = tmp_path / "abi.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "mooncake_ep_hip.h"\n'
+        "int main(void) {\n"
+        '  printf("%zu %zu %zu %zu %zu\\n", sizeof(mc_ep_legacy_perf_tensors_t), sizeof(mc_ep_legacy_perf_config_t),\n'
+        "         offsetof(mc_ep_legacy_perf_config_t, compute_stream_ptr), sizeof(mc_ep_legacy_perf_result_t),\n"
+        "         offsetof(mc_ep_legacy_perf_tensors_t, combined_x_ptrs));\n"
+        "  return (MC_EP_PHASE_ALL == (MC_EP_PHASE_LAYOUT | MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) ? 0 : 1;\n"
+        "}\n")
+    exe = tmp_path / "abi"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    str(src), "-o", str(exe)], check=True, capture_output=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    sizes = [int(v) for v in out]
+    assert sizes == [ctypes.sizeof(_lib.LegacyPerfTensors), ctypes.sizeof(_lib.LegacyPerfConfig),
+                     _lib.LegacyPerfConfig.compute_stream_ptr.offset, ctypes.sizeof(_lib.LegacyPerfResult),
+                     _lib.LegacyPerfTensors.combined_x_ptrs.offset]
