@@ -213,7 +213,9 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "fp8_e4m3 dispatch payload (f32 scale math), bf16 combine with f32 accumulate",
+        "dtype": "f32",
+        "dtype_detail": "bf16 in; fp8 e4m3 payload with f32 scale arithmetic out of dispatch; bf16 rows, f32 "
+                        "accumulation, bf16 out of combine",
         "data": "synthetic",
         "config": {"workload": cfg.name, "num_ranks": cfg.num_ranks, "tokens_per_rank": cfg.tokens_per_rank,
                    "hidden": cfg.hidden, "num_experts": cfg.num_experts, "num_topk": cfg.num_topk,
