@@ -38,8 +38,9 @@ extern "C" {
  * LOW_LATENCY_RECV_PHASE split, mooncake_ep_configs.cuh:16-17, maps onto the
  * kernels each call is made of; a later phase needs the earlier ones of the
  * same call to have run) */
-#define MC_EP_PHASE_LAYOUT 1   /* dispatch: routing layout;  combine: handle -> row resolve */
-#define MC_EP_PHASE_DATA 2     /* dispatch: pack;            combine: weighted reduce */
+#define MC_EP_PHASE_LAYOUT 1   /* dispatch: routing counts;  combine: handle -> row resolve */
+#define MC_EP_PHASE_DATA 2     /* dispatch: pack (packed_recv_count / src_info / layout_range are complete after
+                                  this phase, not before); combine: weighted reduce */
 #define MC_EP_PHASE_FINISH 4   /* dispatch: fp8 scales into their column-major layout; combine: nothing */
 #define MC_EP_PHASE_ALL 7
 
