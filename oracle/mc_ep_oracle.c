@@ -29,6 +29,24 @@
  *   src_info   i32    [R, L, RM]
  *   layout_range i64  [R, L, R]
  *
+ * What pins each function (independently of this file's own formulas); no
+ * function here is "parity unpinned":
+ *   oracle_f32_to_e4m3fn / e4m3fn_to_f32   torch's float8_e4m3fn cast on all 65 536 bf16 values and all 256
+ *                                          codes, OCP known answers            tests/test_oracle_fp8.py
+ *   oracle_f32_to_bf16                     torch's bf16 cast, ties and NaN     tests/test_oracle_fp8.py
+ *   oracle_quantise_rows                   the reference's per_token_cast_to_fp8 (TU:42-47) run by torch,
+ *                                          amax floor, round trip bound        tests/test_oracle_fp8.py
+ *   oracle_layout / oracle_dispatch        brute-force triple loop, bincount closed form, the structured-row
+ *                                          checks of the reference's tests, per-rank torch statement of
+ *                                          PY:787-869, committed fixtures      tests/test_oracle_contract.py,
+ *                                                                              tests/test_golden.py
+ *   oracle_invert_handle / oracle_combine  closed forms x * sum(w) and x * sum(factor * w), float64 gather-sum
+ *                                          within one bf16 ulp, linearity      tests/test_oracle_contract.py
+ *   oracle_cast_back                       per_token_cast_back (TU:50-53) and the grid test's mock expert run
+ *                                          by torch, every fp8 code            tests/test_oracle_cast_back.py
+ *   oracle_buffer_size_hint                the value the reference's layout arithmetic gives for its own
+ *                                          test shapes                         tests/test_abi_exports.py
+ *
  * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off -fopenmp).
  */
 #include <math.h>
