@@ -45,7 +45,7 @@
  *   oracle_cast_back                       per_token_cast_back (TU:50-53) and the grid test's mock expert run
  *                                          by torch, every fp8 code            tests/test_oracle_cast_back.py
  *   oracle_buffer_size_hint                the value the reference's layout arithmetic gives for its own
- *                                          test shapes                         tests/test_abi_exports.py
+ *                                          test shapes                         tests/test_oracle_contract.py
  *
  * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off -fopenmp).
  */
