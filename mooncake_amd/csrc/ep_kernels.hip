@@ -862,6 +862,7 @@ __device__ __forceinline__ uint32_t scale_round_twice(float a, float b, float s,
 // saves every block of the main kernel the same scan (a chain of dependent
 // loads) in front of its first row.
 constexpr int kCastRows = 4;
+constexpr int kCastWaves = 4;        // waves per block of the main kernel: kCastRows / kCastWaves rows each
 constexpr int kCastCols = 1024;
 constexpr int kCastMaxExperts = 4096;
 constexpr int kCastMapBlocks = 8;      // each repeats the scan (cheap) and writes an eighth of the entries
@@ -920,7 +921,7 @@ __global__ __launch_bounds__(1024) void cast_chunks_kernel(const uint64_t* __res
 // are 256 contiguous bytes) are staged in LDS; then each wave converts its 16
 // rows, 16 payload bytes (FP8) or 32 (bf16 payload) per lane and row.
 template <bool FP8>
-__global__ __launch_bounds__(256) void cast_back_kernel(const uint64_t* __restrict__ tbl,
+__global__ __launch_bounds__(kCastWaves * 64) void cast_back_kernel(const uint64_t* __restrict__ tbl,
                                                          const int4* __restrict__ map,
                                                          const float* __restrict__ factor, int R, int E, int H,
                                                          int max_tokens, int parts) {
@@ -963,10 +964,11 @@ __global__ __launch_bounds__(256) void cast_back_kernel(const uint64_t* __restri
                            : nullptr;
     }
 
-    constexpr int kBatch = kCastRows / 4 < 8 ? kCastRows / 4 : 8;   // rows whose loads are in flight together
+    constexpr int kWaveRows = kCastRows / kCastWaves;
+    constexpr int kBatch = kWaveRows < 8 ? kWaveRows : 8;   // rows whose loads are in flight together
     const int64_t row_base = (int64_t)le * RM;
-    for (int b = 0; b < kCastRows / 4; b += kBatch) {
-        const int r_first = row0 + wave * (kCastRows / 4) + b;
+    for (int b = 0; b < kWaveRows; b += kBatch) {
+        const int r_first = row0 + wave * kWaveRows + b;
         if (r_first >= count) break;
         uint4 v[kBatch][2];
         float sv[kBatch][2];
@@ -1242,10 +1244,10 @@ hipError_t launch_cast_back(const uint64_t* d_tbl, void* d_chunk_map, const floa
     hipLaunchKernelGGL(cast_chunks_kernel, dim3(kCastMapBlocks), dim3(1024), 0, stream, d_tbl, map, d.R, d.E, d.max_tokens,
                        (int)chunks);
     if (use_fp8)
-        hipLaunchKernelGGL(cast_back_kernel<true>, dim3((unsigned)total), dim3(256), 0, stream, d_tbl, map, d_factor,
+        hipLaunchKernelGGL(cast_back_kernel<true>, dim3((unsigned)total), dim3(kCastWaves * 64), 0, stream, d_tbl, map, d_factor,
                            d.R, d.E, d.H, d.max_tokens, parts);
     else
-        hipLaunchKernelGGL(cast_back_kernel<false>, dim3((unsigned)total), dim3(256), 0, stream, d_tbl, map, d_factor,
+        hipLaunchKernelGGL(cast_back_kernel<false>, dim3((unsigned)total), dim3(kCastWaves * 64), 0, stream, d_tbl, map, d_factor,
                            d.R, d.E, d.H, d.max_tokens, parts);
     return hipGetLastError();
 }
