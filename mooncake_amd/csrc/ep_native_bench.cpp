@@ -1,0 +1,238 @@
+// A Python-free driver of libmooncake_ep_hip.so: everything it needs from the
+// library is in include/mooncake_ep_hip.h.  It builds a synthetic world in
+// device memory, checks the routing outputs against a host count, and times
+//   * fp8 (or bf16) dispatch + combine steps, whole world, back to back, and
+//   * the library's native loop (the reference's _benchmark_legacy_buffer:
+//     recv_count clear + bf16 dispatch + combine, legacy_buffer_perf.cpp:84-146).
+//
+//   ep_native_bench [--ranks R] [--tokens T] [--hidden H] [--experts E] [--topk K]
+//                   [--bf16] [--warmups W] [--iterations N]
+//
+// Exit status 0 means the self-check passed.  Built by `make bench`.
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "mooncake_ep_hip.h"
+
+namespace {
+
+#define HIP_OK(cmd)                                                                                  \
+    do {                                                                                             \
+        hipError_t e_ = (cmd);                                                                       \
+        if (e_ != hipSuccess) {                                                                      \
+            std::fprintf(stderr, "%s:%d %s: %s\n", __FILE__, __LINE__, #cmd, hipGetErrorString(e_)); \
+            std::exit(2);                                                                            \
+        }                                                                                            \
+    } while (0)
+
+#define EP_OK(cmd)                                                                              \
+    do {                                                                                        \
+        if ((cmd) != MC_EP_OK) {                                                                \
+            std::fprintf(stderr, "%s:%d %s: %s\n", __FILE__, __LINE__, #cmd, mc_ep_last_error()); \
+            std::exit(2);                                                                       \
+        }                                                                                       \
+    } while (0)
+
+struct Args {
+    int ranks = 32, tokens = 128, hidden = 7168, experts = 256, topk = 8, warmups = 20, iterations = 30;
+    bool fp8 = true;
+};
+
+Args parse(int argc, char** argv) {
+    Args a;
+    for (int i = 1; i < argc; ++i) {
+        const std::string f = argv[i];
+        auto value = [&]() -> int {
+            if (i + 1 >= argc) {
+                std::fprintf(stderr, "%s needs a value\n", f.c_str());
+                std::exit(2);
+            }
+            return std::atoi(argv[++i]);
+        };
+        if (f == "--ranks") a.ranks = value();
+        else if (f == "--tokens") a.tokens = value();
+        else if (f == "--hidden") a.hidden = value();
+        else if (f == "--experts") a.experts = value();
+        else if (f == "--topk") a.topk = value();
+        else if (f == "--warmups") a.warmups = value();
+        else if (f == "--iterations") a.iterations = value();
+        else if (f == "--bf16") a.fp8 = false;
+        else {
+            std::fprintf(stderr, "unknown flag %s\n", f.c_str());
+            std::exit(2);
+        }
+    }
+    if (a.ranks < 1 || a.experts % a.ranks || a.hidden % 128 || a.topk < 1 || a.topk > a.experts || a.tokens < 1 ||
+        a.iterations < 2 || (a.fp8 && ((long long)a.ranks * a.tokens) % 4)) {
+        std::fprintf(stderr, "unusable shape\n");
+        std::exit(2);
+    }
+    return a;
+}
+
+// xorshift: a reproducible stream that needs no library
+struct Rng {
+    uint64_t s;
+    explicit Rng(uint64_t seed) : s(seed * 0x9E3779B97F4A7C15ull + 1) {}
+    uint64_t next() {
+        s ^= s << 13;
+        s ^= s >> 7;
+        s ^= s << 17;
+        return s;
+    }
+    float unit() { return (float)((next() >> 40) & 0xFFFFFF) / 16777216.0f; }
+};
+
+uint16_t to_bf16(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+template <typename T>
+T* device_copy(const std::vector<T>& host) {
+    T* d = nullptr;
+    HIP_OK(hipMalloc((void**)&d, host.size() * sizeof(T)));
+    HIP_OK(hipMemcpy(d, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice));
+    return d;
+}
+
+template <typename T>
+std::vector<uint64_t> per_rank(const T* base, size_t stride_elems, int ranks) {
+    std::vector<uint64_t> p((size_t)ranks);
+    for (int r = 0; r < ranks; ++r) p[(size_t)r] = (uint64_t)(base + (size_t)r * stride_elems);
+    return p;
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+    const Args a = parse(argc, argv);
+    const int R = a.ranks, T = a.tokens, H = a.hidden, E = a.experts, K = a.topk, L = E / R;
+    const size_t RM = (size_t)R * T;
+
+    // inputs: x ~ uniform(-1, 1) as bf16; top-k = K distinct experts per token; weights sum to one
+    std::vector<uint16_t> hx((size_t)R * T * H);
+    std::vector<int64_t> hidx((size_t)R * T * K);
+    std::vector<float> hw((size_t)R * T * K);
+    std::vector<long long> expect((size_t)E, 0);
+    Rng rng(2026);
+    for (auto& v : hx) v = to_bf16(rng.unit() * 2.0f - 1.0f);
+    std::vector<int> pool((size_t)E);
+    for (size_t n = 0; n < (size_t)R * T; ++n) {
+        for (int e = 0; e < E; ++e) pool[(size_t)e] = e;
+        float wsum = 0.0f;
+        for (int k = 0; k < K; ++k) {   // partial Fisher-Yates: K distinct experts
+            const int j = k + (int)(rng.next() % (uint64_t)(E - k));
+            std::swap(pool[(size_t)k], pool[(size_t)j]);
+            hidx[n * K + k] = pool[(size_t)k];
+            expect[(size_t)pool[(size_t)k]]++;
+            hw[n * K + k] = 0.1f + rng.unit();
+            wsum += hw[n * K + k];
+        }
+        for (int k = 0; k < K; ++k) hw[n * K + k] /= wsum;
+    }
+
+    uint16_t* x = device_copy(hx);
+    int64_t* idx = device_copy(hidx);
+    float* wts = device_copy(hw);
+    std::vector<int32_t> ones((size_t)R * R, 1);
+    int32_t* active = device_copy(ones);
+    const size_t payload = a.fp8 ? 1 : 2;
+    uint8_t* recv_x = nullptr;
+    float* scales = nullptr;
+    uint16_t *recv_bf16 = nullptr, *expert_x = nullptr, *out = nullptr;
+    int32_t *recv_count = nullptr, *src_info = nullptr;
+    int64_t* layout_range = nullptr;
+    HIP_OK(hipMalloc((void**)&recv_x, (size_t)R * L * RM * H * payload));
+    if (a.fp8) HIP_OK(hipMalloc((void**)&scales, (size_t)R * L * (H / 128) * RM * sizeof(float)));
+    HIP_OK(hipMalloc((void**)&recv_bf16, (size_t)R * L * RM * H * 2));     // the native loop's bf16 receive layout
+    HIP_OK(hipMalloc((void**)&expert_x, (size_t)R * L * RM * H * 2));
+    HIP_OK(hipMemset(expert_x, 0, (size_t)R * L * RM * H * 2));
+    HIP_OK(hipMalloc((void**)&out, (size_t)R * T * H * 2));
+    HIP_OK(hipMalloc((void**)&recv_count, (size_t)R * L * sizeof(int32_t)));
+    HIP_OK(hipMalloc((void**)&src_info, (size_t)R * L * RM * sizeof(int32_t)));
+    HIP_OK(hipMalloc((void**)&layout_range, (size_t)R * L * R * sizeof(int64_t)));
+
+    const auto px = per_rank(x, (size_t)T * H, R), pidx = per_rank(idx, (size_t)T * K, R);
+    const auto pw = per_rank(wts, (size_t)T * K, R), pact = per_rank(active, (size_t)R, R);
+    const auto precv = per_rank(recv_x, (size_t)L * RM * H * payload, R);
+    const auto pscales = a.fp8 ? per_rank(scales, (size_t)L * (H / 128) * RM, R) : std::vector<uint64_t>();
+    const auto precv16 = per_rank(recv_bf16, (size_t)L * RM * H, R), pexp = per_rank(expert_x, (size_t)L * RM * H, R);
+    const auto pout = per_rank(out, (size_t)T * H, R), pcnt = per_rank(recv_count, (size_t)L, R);
+    const auto psrc = per_rank(src_info, (size_t)L * RM, R), plr = per_rank(layout_range, (size_t)L * R, R);
+    const std::vector<int32_t> tokens((size_t)R, T);
+
+    mc_ep_world_t* world = nullptr;
+    EP_OK(mc_ep_world_create(R, &world));
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    const uint64_t s = (uint64_t)stream;
+
+    auto dispatch = [&] {
+        EP_OK(mc_ep_world_dispatch(world, px.data(), pidx.data(), tokens.data(), H, K, T, E, a.fp8 ? 1 : 0, precv.data(),
+                                   a.fp8 ? pscales.data() : nullptr, pcnt.data(), psrc.data(), plr.data(),
+                                   MC_EP_PHASE_ALL, s));
+    };
+    auto combine = [&] {
+        EP_OK(mc_ep_world_combine(world, pexp.data(), pidx.data(), pw.data(), psrc.data(), plr.data(), pact.data(),
+                                  tokens.data(), H, K, T, E, pout.data(), MC_EP_PHASE_ALL, s));
+    };
+
+    // self-check: every expert received exactly the rows that name it
+    dispatch();
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<int32_t> got((size_t)E);
+    HIP_OK(hipMemcpy(got.data(), recv_count, (size_t)E * sizeof(int32_t), hipMemcpyDeviceToHost));
+    for (int e = 0; e < E; ++e) {
+        if (got[(size_t)e] != expect[(size_t)e]) {
+            std::fprintf(stderr, "self-check failed: expert %d received %d rows, %lld selections name it\n", e,
+                         got[(size_t)e], expect[(size_t)e]);
+            return 1;
+        }
+    }
+    // the mock expert of the reference's tests, on valid rows only
+    EP_OK(mc_ep_world_cast_back(world, precv.data(), a.fp8 ? pscales.data() : nullptr, pcnt.data(), 0, pexp.data(), H, K,
+                                T, E, s));
+
+    for (int i = 0; i < a.warmups; ++i) {
+        dispatch();
+        combine();
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < a.iterations; ++i) {
+        dispatch();
+        combine();
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    const double step_us =
+        std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count() / a.iterations;
+
+    const double N = (double)R * T, S = N * K;
+    const double row = a.fp8 ? H + H / 128 * 4.0 : 2.0 * H;
+    const double bytes = N * H * 2 + N * K * 8 + S * (row + 4) + E * 4.0 + (double)E * R * 8   // dispatch
+                         + S * H * 2 + N * K * 12 + S * 4 + N * H * 2;                          // combine
+    std::printf("%s dispatch + combine, %d ranks x %d tokens, hidden %d, %d experts, top-%d: %.1f us per step, "
+                "%.0f GB/s (%.1f %% of 8 TB/s)\n",
+                a.fp8 ? "fp8" : "bf16", R, T, H, E, K, step_us, bytes / step_us / 1e3, bytes / step_us / 1e3 / 80.0);
+
+    mc_ep_legacy_perf_tensors_t lt = {px.data(),      pidx.data(), pw.data(),  pact.data(), pexp.data(),
+                                      precv16.data(), pcnt.data(), psrc.data(), plr.data(),  pout.data()};
+    mc_ep_legacy_perf_config_t lc = {T, H, K, L, T, E, -1, a.warmups, a.iterations, s};
+    mc_ep_legacy_perf_result_t lr = {0, 0, 0};
+    EP_OK(mc_ep_world_legacy_buffer_perf(world, &lt, &lc, &lr));
+    std::printf("native loop (clear + bf16 dispatch + combine): avg_t=%.2f us, min_t=%.2f us, max_t=%.2f us\n",
+                lr.average_us, lr.min_us, lr.max_us);
+
+    EP_OK(mc_ep_world_destroy(world));
+    HIP_OK(hipStreamDestroy(stream));
+    return 0;
+}

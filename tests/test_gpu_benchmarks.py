@@ -128,3 +128,23 @@ def test_ep_benchmark_zero_copy_is_refused_like_the_reference_build_without_it(g
     bench = runner.EPBenchmark(_bench_args("--zero-copy"))
     with pytest.raises(NotImplementedError):
         bench.cycle()
+
+
+def test_native_driver_runs_without_python_in_the_loop(gpu_device):
+    """The C++ driver built from the C header alone: self-check (per-expert row counts against a host count)
+    and both timing loops."""
+    import os
+    import subprocess
+    from mooncake_amd import _lib
+    exe = os.path.join(os.path.dirname(_lib.LIB_PATH), "ep_native_bench")
+    assert os.path.exists(exe), "build it first (make -C mooncake_amd/csrc)"
+    announce("native driver")
+    for flags in (["--ranks", "4", "--tokens", "32", "--hidden", "1024", "--experts", "16", "--topk", "4",
+                   "--warmups", "2", "--iterations", "4"],
+                  ["--ranks", "2", "--tokens", "17", "--hidden", "256", "--experts", "6", "--topk", "3", "--bf16",
+                   "--warmups", "1", "--iterations", "3"]):
+        run = subprocess.run([exe] + flags, capture_output=True, text=True, timeout=100)
+        assert run.returncode == 0, run.stderr
+        assert "us per step" in run.stdout and "native loop" in run.stdout
+    bad = subprocess.run([exe, "--ranks", "3", "--experts", "16"], capture_output=True, text=True, timeout=100)
+    assert bad.returncode == 2 and "unusable shape" in bad.stderr
