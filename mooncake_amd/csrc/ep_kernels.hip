@@ -924,14 +924,21 @@ template <bool FP8>
 __global__ __launch_bounds__(kCastWaves * 64) void cast_back_kernel(const uint64_t* __restrict__ tbl,
                                                          const int4* __restrict__ map,
                                                          const float* __restrict__ factor, int R, int E, int H,
-                                                         int max_tokens, int parts) {
+                                                         int max_tokens, int parts, int max_chunks) {
     const int lane = wave_lane();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int target = blockIdx.x / parts, part = blockIdx.x - target * parts;
+    // Blocks go round-robin over the 8 XCDs, each with an L2 of its own.  The four chunks that share
+    // 64-byte sectors of scales (16 consecutive rows of one group) are therefore given to four blocks
+    // of the same XCD, next to each other in launch order: block = (set / 8 * 4 + chunk % 4) * 8 + set % 8,
+    // with set = (chunk / 4) * parts + part.
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int set = (seq >> 2) * 8 + xcd;
+    const int part = set % parts;
+    const int target = (set / parts) * 4 + (seq & 3);
     const int L = E / R;
     const int64_t RM = (int64_t)R * max_tokens;
     const int total = map[0].x;
-    const int4 item = map[1 + target];      // in bounds: the map holds an entry per possible chunk
+    const int4 item = map[1 + (target < max_chunks ? target : 0)];
     if (target >= total) return;            // block-uniform
     const int e = __builtin_amdgcn_readfirstlane(item.x);
     const int chunk = __builtin_amdgcn_readfirstlane(item.y);
@@ -1243,12 +1250,16 @@ hipError_t launch_cast_back(const uint64_t* d_tbl, void* d_chunk_map, const floa
     int4* map = (int4*)d_chunk_map;
     hipLaunchKernelGGL(cast_chunks_kernel, dim3(kCastMapBlocks), dim3(1024), 0, stream, d_tbl, map, d.R, d.E, d.max_tokens,
                        (int)chunks);
+    // sets of four chunks times parts, rounded up to whole rounds over the 8 XCDs
+    const long long sets = (chunks + 3) / 4 * parts;
+    const long long blocks = (sets + 7) / 8 * 8 * 4;
+    if (blocks > 0x7fffffffll) return hipErrorInvalidValue;
     if (use_fp8)
-        hipLaunchKernelGGL(cast_back_kernel<true>, dim3((unsigned)total), dim3(kCastWaves * 64), 0, stream, d_tbl, map, d_factor,
-                           d.R, d.E, d.H, d.max_tokens, parts);
+        hipLaunchKernelGGL(cast_back_kernel<true>, dim3((unsigned)blocks), dim3(kCastWaves * 64), 0, stream, d_tbl, map,
+                           d_factor, d.R, d.E, d.H, d.max_tokens, parts, (int)chunks);
     else
-        hipLaunchKernelGGL(cast_back_kernel<false>, dim3((unsigned)total), dim3(kCastWaves * 64), 0, stream, d_tbl, map, d_factor,
-                           d.R, d.E, d.H, d.max_tokens, parts);
+        hipLaunchKernelGGL(cast_back_kernel<false>, dim3((unsigned)blocks), dim3(kCastWaves * 64), 0, stream, d_tbl,
+                           map, d_factor, d.R, d.E, d.H, d.max_tokens, parts, (int)chunks);
     return hipGetLastError();
 }
 
