@@ -2,6 +2,7 @@
 counts (some zero), masked tokens, ranks that take no part, per-rank views of
 inactive ranks.  Every case runs dispatch -> cast back -> combine through the C
 ABI and is compared with the oracle bit for bit."""
+import os
 import random
 
 import pytest
@@ -40,7 +41,8 @@ def _case(seed: int):
     return cfg, num_tokens, present, active, direct, summed
 
 
-@pytest.mark.parametrize("seed", range(32))
+# more seeds for a longer sweep: MC_EP_RANDOM_WORLDS=300 python -m pytest tests/test_gpu_random_shapes.py -m gpu
+@pytest.mark.parametrize("seed", range(int(os.environ.get("MC_EP_RANDOM_WORLDS", "32"))))
 def test_random_world(gpu_device, oracle, seed):
     cfg, num_tokens, present, active, direct, summed = _case(seed)
     announce(f"random world seed={seed} {cfg} tokens={num_tokens} present={present} direct={direct} summed={summed}")
