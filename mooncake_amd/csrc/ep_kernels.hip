@@ -3,11 +3,13 @@
 // payload access is a 16-byte vector load or store that a wave issues over a
 // contiguous span of a row.
 //
-//   count_kernel,   routing layout: per-expert histogram of every unit of 256
-//   prefix_kernel   selections, position of each selection inside it, exclusive
-//                   prefix over units, per-(expert, source rank) ranges and
-//                   per-expert counts.  Restates the count path and the slot
-//                   assignment of the reference's dispatch
+//   count_kernel,   routing layout: per-expert histogram of every unit of 1024
+//   prefix pass     (or 256) selections, position of each selection inside it,
+//                   exclusive prefix over units, per-(expert, source rank)
+//                   ranges and per-expert counts.  The prefix pass runs as the
+//                   first waves of the pack launch (summed plan) or as
+//                   prefix_kernel (table plan).  Restates the count path and
+//                   the slot assignment of the reference's dispatch
 //                   (mooncake-ep/src/mooncake_ep_kernel.cu:274, :319-356,
 //                   :417-437) in a deterministic order: source rank ascending,
 //                   token ascending, as the reference's PyTorch statement has
@@ -26,6 +28,10 @@
 //   reduce_kernel   per token: fp32 fused multiply-add over its top-k expert
 //                   rows in k order, round to nearest even bf16
 //                   (mooncake_ep_kernel.cu:711-753).
+//   cast_chunks_kernel,  the consumer of the packed layout: valid rows back to
+//   cast_back_kernel     bf16, times a per-expert factor
+//                   (per_token_cast_back, mooncake-wheel/tests/ep_test_utils.py:50-53;
+//                   the mock expert of mooncake-ep/tests/test_ep_grid.py:168-173).
 #include "ep_kernels.h"
 
 namespace mcep {
