@@ -27,6 +27,9 @@ SMALL = [
     EPConfig("experts768", 8, 16, 256, 768, 8, True),
     EPConfig("experts1024", 8, 16, 256, 1024, 8, False),
     EPConfig("units80", 16, 600, 256, 32, 8, False),
+    # more ranks than one table-writer launch carries (384 words): the rank table goes up in pieces
+    EPConfig("ranks64", 64, 4, 128, 64, 2, True),
+    EPConfig("ranks100", 100, 3, 128, 100, 3, False),
 ]
 
 
