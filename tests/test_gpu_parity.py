@@ -153,6 +153,7 @@ COMBINE_CASES = [
     EPConfig("k16_c", 2, 20, 1024, 32, 16, False),
     EPConfig("masked_c", 8, 64, 1024, 8, 2, False, masked_fraction=0.3),
     EPConfig("fp8_c", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05),
+    EPConfig("ranks64_c", 64, 4, 128, 64, 2, True),                  # rank table in two pieces
     shrink(CONFIGS["cpu_check"]),
 ]
 
