@@ -88,6 +88,27 @@ def time_pipeline(h, lib, iters, flush=None):
     return out
 
 
+def time_calls(h, iters, flush=None):
+    """Device time of a whole dispatch and a whole combine inside the running pipeline: three events per
+    step (start, between, end), so each figure carries one marker's overhead instead of one per kernel."""
+    import torch
+    marks = []
+    for _ in range(iters + 2):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        if flush is not None:
+            flush.zero_()
+        ev[0].record()
+        h.dispatch()
+        ev[1].record()
+        h.combine()
+        ev[2].record()
+        marks.append(ev)
+    torch.cuda.synchronize()
+    d = [m[0].elapsed_time(m[1]) * 1e3 for m in marks[2:]]
+    c = [m[1].elapsed_time(m[2]) * 1e3 for m in marks[2:]]
+    return sum(d) / len(d), sum(c) / len(c)
+
+
 def cpu_baseline(cfg, data, bytes_total, budget_s):
     """The oracle (a scalar C restatement, OpenMP over tokens) timed on this
     host's cores on the same workload: whole steps until the budget is spent."""
@@ -185,8 +206,7 @@ def main():
     # per-kernel device times, measured live inside the pipeline
     flush = torch.empty(args.flush_mb << 20, dtype=torch.uint8, device="cuda:0") if args.flush_mb > 0 else None
     t = time_pipeline(h, _lib, args.kernel_iters, flush)
-    d_us = sum(t[k][0] for k in ("layout", "pack", "scales") if k in t)
-    c_us = sum(t[k][0] for k in ("resolve", "reduce") if k in t)
+    d_us, c_us = time_calls(h, args.kernel_iters, flush)
     pack_us, red_us = t["pack"][0], t["reduce"][0]
     kernels = {k: {"us": round(v[0], 2), "min_us": round(v[1], 2)} for k, v in t.items()}
     kernels["pack"].update(bytes=alg["dispatch"], GBps=round(alg["dispatch"] / pack_us / 1e3, 1))
