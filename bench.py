@@ -109,6 +109,22 @@ def time_calls(h, iters, flush=None):
     return sum(d) / len(d), sum(c) / len(c)
 
 
+def time_back_to_back(call, iters):
+    """Average launch period of one kernel: `iters` launches of it in a row between one event pair, so the
+    markers' own overhead (2-3 us each) is spread over all of them.  This is the figure a profiler's kernel
+    duration corresponds to (end of the previous kernel to end of this one)."""
+    import torch
+    for _ in range(3):
+        call()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        call()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / iters
+
+
 def cpu_baseline(cfg, data, bytes_total, budget_s):
     """The oracle (a scalar C restatement, OpenMP over tokens) timed on this
     host's cores on the same workload: whole steps until the budget is spent."""
@@ -211,6 +227,15 @@ def main():
     kernels = {k: {"us": round(v[0], 2), "min_us": round(v[1], 2)} for k, v in t.items()}
     kernels["pack"].update(bytes=alg["dispatch"], GBps=round(alg["dispatch"] / pack_us / 1e3, 1))
     kernels["reduce"].update(bytes=alg["combine"], GBps=round(alg["combine"] / red_us / 1e3, 1))
+    # the two data kernels once more, each launched back to back (see time_back_to_back): reported beside
+    # the in-pipeline durations, which carry a marker's overhead each and are the ones the roofline uses
+    h.dispatch()
+    pack_b2b = time_back_to_back(lambda: h.dispatch(phases=_lib.PHASE_DATA), args.kernel_iters)
+    direct = bool(h.world.get_option("combine_direct"))
+    red_b2b = time_back_to_back(lambda: h.combine(phases=_lib.PHASE_ALL if direct else _lib.PHASE_DATA),
+                                args.kernel_iters)
+    kernels["pack"].update(us_back_to_back=round(pack_b2b, 2))
+    kernels["reduce"].update(us_back_to_back=round(red_b2b, 2))
     # the consumer of the packed layout (valid rows -> bf16), outside the step: reported, not part of `value`
     H = cfg.hidden
     cast_bytes = S * ((H + H // 128 * 4) if cfg.use_fp8 else 2 * H) + S * 2 * H
