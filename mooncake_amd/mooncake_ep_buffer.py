@@ -88,14 +88,14 @@ class Buffer:
         self._keepalive = collections.deque(maxlen=4)
         self.connect()
 
-    def connect(self, active_ranks=None) -> None:
-        """Peer exchange of the reference (:185-304) has nothing to do when
-        every rank lives in the same address space."""
+    def connect(self, is_update: bool = False) -> None:
+        """Peer exchange of the reference (:185-304; is_update re-runs it for a changed membership, :306-307)
+        has nothing to do when every rank lives in the same address space."""
         if not self.runtime.use_fast_path():
             raise RuntimeError("mooncake_amd has no fallback path")
 
     def update_ep_member(self) -> None:
-        self.connect(True)
+        self.connect(is_update=True)
 
     @staticmethod
     def get_ep_buffer_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
