@@ -317,7 +317,7 @@ ORACLE_API void oracle_combine(int R, int E, int K, int Tmax, int max_tokens, in
             for (int j = 0; j < H; ++j) acc[j] = 0.0f;
             for (int k = 0; k < K; ++k) {
                 const int64_t e = topk_idx[n * K + k];
-                if (e < 0) continue;
+                if (e < 0 || e >= E) continue;   /* ids outside [0, E) name no expert */
                 if (active && !active[(int64_t)r * R + e / L]) continue;
                 const int slot = slot_map[n * K + k];
                 if (slot < 0) continue;

@@ -250,3 +250,37 @@ def test_dispatch_with_silent_rank(gpu_device, oracle):
     h.recv_count[2] = 0
     ref["recv_count"][2] = 0
     compare_dispatch(h, ref, check_poison=False)
+
+
+@pytest.mark.parametrize("direct", [1, 0])
+def test_ids_outside_the_expert_range_name_no_expert(gpu_device, oracle, direct):
+    """The reference asserts nothing about top-k ids; here anything outside [0, E) is treated like -1 by every
+    kernel (and by the oracle), instead of indexing out of bounds."""
+    cfg = EPConfig("stray_ids", 4, 24, 512, 8, 4, True)
+    announce(f"stray expert ids direct={direct}")
+    data = generate(cfg, seed=9)
+    idx = data["topk_idx"]
+    gen = torch.Generator().manual_seed(1)
+    stray = torch.rand(idx.shape, generator=gen)
+    idx[stray < 0.1] = cfg.num_experts + 3
+    idx[(stray >= 0.1) & (stray < 0.2)] = -5
+    idx[(stray >= 0.2) & (stray < 0.25)] = 2 ** 40
+    clean = idx.clone()
+    clean[(idx < 0) | (idx >= cfg.num_experts)] = -1
+    h = run_dispatch(cfg, data, poison=True, options={"combine_direct": direct})
+    nt = [cfg.tokens_per_rank] * cfg.num_ranks
+    ref = oracle.dispatch(data["x"], idx, nt, cfg.max_tokens, cfg.num_experts, True)
+    same = oracle.dispatch(data["x"], clean, nt, cfg.max_tokens, cfg.num_experts, True)
+    assert torch.equal(ref["recv_count"], same["recv_count"]) and torch.equal(ref["layout_range"], same["layout_range"])
+    compare_dispatch(h, ref, check_poison=True)
+    h.alloc_combine_io()
+    h.cast_back(None)
+    h.combine()
+    torch.cuda.synchronize()
+    rows = oracle.cast_back(ref["recv_x"], ref["scales"], ref["recv_count"], None)
+    want = oracle.combine(rows, idx, data["topk_weights"], ref["src_info"], ref["layout_range"], nt, cfg.max_tokens,
+                          cfg.num_experts)
+    want_clean = oracle.combine(rows, clean, data["topk_weights"], ref["src_info"], ref["layout_range"], nt,
+                                cfg.max_tokens, cfg.num_experts)
+    assert torch.equal(want.view(torch.int16), want_clean.view(torch.int16))
+    assert torch.equal(h.combined.cpu().view(torch.int16), want.view(torch.int16))
