@@ -97,6 +97,30 @@ int mc_ep_world_dispatch(mc_ep_world_t* world, const uint64_t* x_ptrs, const uin
                          const uint64_t* packed_recv_count_ptrs, const uint64_t* packed_recv_src_info_ptrs,
                          const uint64_t* packed_recv_layout_range_ptrs, int phases, uint64_t stream_ptr);
 
+/* mc_ep_world_dispatch (all phases) for callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It has no counterpart in the reference.  The call makes no
+ * hipMalloc / hipFree and no other allocating call, whatever the shape: the
+ * routing state, the fp8 scale staging rows and the rank table live in a
+ * 16 MiB array in static device memory that each GPU the library runs on holds
+ * until the process ends.  A shape that needs more (about
+ * num_experts * num_ranks * max_tokens * 4 bytes, plus
+ * num_ranks * max_tokens * (num_topk * 4 + hidden / 32) bytes) is rejected with
+ * MC_EP_ERR_ASSERT and a message that says so; the DeepSeek-V3 decode world
+ * (32 x 128 tokens, 256 experts, hidden 7168) needs 5.3 MB.  Same arguments,
+ * outputs and errors as mc_ep_world_dispatch otherwise.  Every call on a GPU,
+ * from any world, shares that GPU's array and overwrites the last call's
+ * contents: calls that overlap on one GPU (different streams without an order
+ * between them, or different threads) race.  A combine given this dispatch's
+ * handle reads src_info / layout_range as any combine of an older handle does
+ * (it does not find the routing state of "the last dispatch"). */
+int mc_ep_world_dispatch_noalloc(mc_ep_world_t* world, const uint64_t* x_ptrs, const uint64_t* topk_idx_ptrs,
+                                 const int32_t* num_tokens, int hidden, int num_topk,
+                                 int num_max_dispatch_tokens_per_rank, int num_experts, int use_fp8,
+                                 const uint64_t* packed_recv_x_ptrs, const uint64_t* packed_recv_x_scales_ptrs,
+                                 const uint64_t* packed_recv_count_ptrs, const uint64_t* packed_recv_src_info_ptrs,
+                                 const uint64_t* packed_recv_layout_range_ptrs, uint64_t stream_ptr);
+
 /* Whole-world combine: every rank's MooncakeEpBuffer::combine
  * (mooncake_ep_buffer.h:126-133, mooncake_ep_buffer.cpp:341-474).
  *   x [E/R, R*max, hidden] bf16 (expert outputs held by the rank; 0: the rank

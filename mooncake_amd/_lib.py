@@ -54,6 +54,8 @@ SIGNATURES = {
     "mc_ep_world_get_option": (c_int, [c_void_p, c_char_p, POINTER(c_int)]),
     "mc_ep_world_dispatch": (c_int, [c_void_p, _U64P, _U64P, _I32P, c_int, c_int, c_int, c_int, c_int,
                                      _U64P, _U64P, _U64P, _U64P, _U64P, c_int, c_uint64]),
+    "mc_ep_world_dispatch_noalloc": (c_int, [c_void_p, _U64P, _U64P, _I32P, c_int, c_int, c_int, c_int, c_int,
+                                             _U64P, _U64P, _U64P, _U64P, _U64P, c_uint64]),
     "mc_ep_world_combine": (c_int, [c_void_p, _U64P, _U64P, _U64P, _U64P, _U64P, _U64P, _I32P, c_int, c_int,
                                     c_int, c_int, _U64P, c_int, c_uint64]),
     "mc_ep_world_cast_back": (c_int, [c_void_p, _U64P, _U64P, _U64P, c_uint64, _U64P, c_int, c_int, c_int, c_int,

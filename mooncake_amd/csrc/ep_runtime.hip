@@ -19,7 +19,18 @@
 
 using namespace mcep;
 
+// Scratch of the allocation-free dispatch (mc_ep_world_dispatch_noalloc): the routing state, the fp8
+// scale staging rows and the rank table of one call, carved out of one array that every GPU the
+// library runs on holds until the process ends.  Host code never passes the array's name to a
+// kernel: the device address is fetched once per device with hipGetSymbolAddress (world creation)
+// and kept in g_scratch_ptr.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};
 
 thread_local std::string g_last_error;
 
@@ -335,7 +346,8 @@ RoutingScratch routing_scratch(const mc_ep_world* w) {
 int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_idx, const int32_t* num_tokens,
                         int hidden, int num_topk, int max_tokens, int num_experts, int use_fp8,
                         const uint64_t* recv_x, const uint64_t* recv_scales, const uint64_t* recv_count,
-                        const uint64_t* src_info, const uint64_t* layout_range, int phases, hipStream_t stream) {
+                        const uint64_t* src_info, const uint64_t* layout_range, int phases, hipStream_t stream,
+                        bool static_scratch = false) {
     const int R = w->R;
     if (int rc = check_dims(w, hidden, num_topk, max_tokens, num_experts)) return rc;
     MC_ASSERT(x != nullptr && topk_idx != nullptr && num_tokens != nullptr);
@@ -345,7 +357,9 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         MC_ASSERT(recv_scales != nullptr);
     }
     int tgrid = 0;
-    std::vector<uint64_t> tbl((size_t)DF_COUNT * R, 0);
+    // the rank table: on the stack, so that the allocation-free variant touches no heap either
+    uint64_t tbl[(size_t)DF_COUNT * MC_EP_MAX_QP_COUNT];
+    const size_t tbl_words = (size_t)DF_COUNT * R;
     for (int r = 0; r < R; ++r) {
         MC_ASSERT(num_tokens[r] >= 0 && num_tokens[r] <= max_tokens);
         MC_ASSERT(num_tokens[r] == 0 || (x[r] != 0 && topk_idx[r] != 0));
@@ -364,55 +378,89 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         if (num_tokens[r] > tgrid) tgrid = num_tokens[r];
     }
     DeviceGuard guard(w->device);
-    Capture cap;
-    if (int rc = capture_of(stream, &cap)) return rc;
-    RecordingScope recording(cap.active);
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
     plan_units(d, w->tuning);
     // the count kernel keeps per-wave counts and prefixes of every expert in LDS
     MC_ASSERT(count_lds_bytes(d) <= kMaxCountLdsBytes);
     MC_ASSERT(d.units() <= kMaxUnits);
     const size_t UE = (size_t)d.units() * num_experts;
-    if (int rc = ensure_scratch(&w->d_ucount, &w->ucount_cap, UE)) return rc;
-    if (int rc = ensure_scratch(&w->d_ubegin, &w->ubegin_cap, UE)) return rc;
-    if (int rc = ensure_scratch(&w->d_ucount_t, &w->ucount_t_cap, (size_t)num_experts * kMaxSummedUnits)) return rc;
-    if (int rc = ensure_scratch(&w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
-    if (int rc = ensure_scratch(&w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
-    if (int rc = ensure_scratch(&w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
-    if (int rc = ensure_scratch(&w->d_ticket, &w->ticket_cap, (size_t)1)) return rc;
+    const size_t stage_floats = use_fp8 ? (size_t)R * max_tokens * (hidden / 128) : 0;
+
+    RoutingScratch sc{};
+    float* stage = nullptr;
     const uint64_t* d_tbl = nullptr;
-    if (int rc = upload_table(w, 0, tbl, cap, stream, &d_tbl)) return rc;
+    Capture cap;
+    if (static_scratch) {
+        // every piece comes out of the device's static array; nothing is allocated, whatever the shape
+        unsigned char* base = (w->device >= 0 && w->device < kMaxDevices) ? g_scratch_ptr[w->device] : nullptr;
+        MC_ASSERT(base != nullptr);
+        size_t used = 0;
+        auto carve = [&](size_t bytes) {
+            unsigned char* p = base + used;
+            used += (bytes + 255) & ~(size_t)255;
+            return p;
+        };
+        uint64_t* s_tbl = (uint64_t*)carve(tbl_words * sizeof(uint64_t));
+        sc.ucount = (int32_t*)carve(UE * 4);
+        sc.ucount_t = (int32_t*)carve((size_t)num_experts * kMaxSummedUnits * 4);
+        sc.ubegin = (int32_t*)carve(UE * 4);
+        sc.selpos = (int32_t*)carve((size_t)R * max_tokens * num_topk * 4);
+        sc.counts = (int32_t*)carve((size_t)num_experts * 4);
+        sc.row_src = (int32_t*)carve((size_t)num_experts * R * max_tokens * 4);
+        stage = (float*)carve(stage_floats * 4);
+        if (used > kStaticScratchBytes)
+            return fail(MC_EP_ERR_ASSERT,
+                        "Failed: this shape needs " + std::to_string(used) + " bytes of scratch; the allocation-free "
+                        "dispatch holds " + std::to_string(kStaticScratchBytes) + " (use mc_ep_world_dispatch)");
+        // the table travels in kernel arguments on the call's own stream, every time: a recorded call
+        // then carries its own copy, and nothing of the world's eager state is involved
+        MC_HIP(launch_table_write(s_tbl, tbl, (int)tbl_words, stream));
+        d_tbl = s_tbl;
+        // the world's own routing state is no longer that of "the last dispatch": combines resolve their handle
+        w->last.valid = false;
+    } else {
+        if (int rc = capture_of(stream, &cap)) return rc;
+        RecordingScope recording(cap.active);
+        if (int rc = ensure_scratch(&w->d_ucount, &w->ucount_cap, UE)) return rc;
+        if (int rc = ensure_scratch(&w->d_ubegin, &w->ubegin_cap, UE)) return rc;
+        if (int rc = ensure_scratch(&w->d_ucount_t, &w->ucount_t_cap, (size_t)num_experts * kMaxSummedUnits)) return rc;
+        if (int rc = ensure_scratch(&w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
+        if (int rc = ensure_scratch(&w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
+        if (int rc = ensure_scratch(&w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
+        if (stage_floats > 0 && (phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
+            if (int rc = ensure_scale_stage(w, stage_floats)) return rc;
+            stage = w->d_scale_stage;
+        }
+        const std::vector<uint64_t> tbl_vec(tbl, tbl + tbl_words);
+        if (int rc = upload_table(w, 0, tbl_vec, cap, stream, &d_tbl)) return rc;
+        sc = routing_scratch(w);
+    }
 
     const bool uni = w->tuning.uniform != 0;
     DispatchSource src;
     src.x = uniform_ptr(x, R, uni);
     src.topk_idx = uniform_ptr(topk_idx, R, uni);
     src.tokens = uniform_tokens(num_tokens, R, uni);
-    const RoutingScratch sc = routing_scratch(w);
     if (phases & MC_EP_PHASE_LAYOUT) {
         MC_HIP(launch_count(d_tbl, sc, src, d, stream));
-        auto& ld = w->last;
-        ld.valid = true;
-        ld.hidden = hidden; ld.num_topk = num_topk; ld.max_tokens = max_tokens; ld.num_experts = num_experts;
-        ld.topk_idx.assign(topk_idx, topk_idx + R);
-        ld.recv_x.assign(recv_x, recv_x + R);
-        ld.src_info.assign(src_info, src_info + R);
-        ld.layout_range.assign(layout_range, layout_range + R);
-        ld.num_tokens.assign(num_tokens, num_tokens + R);
-        ld.plan = d.plan;
-        ld.captured = cap.active;
-        ld.capture_id = cap.id;
-        if (cap.active) w->dispatch_captured = true;
-    }
-    if ((phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
-        float* stage = nullptr;
-        if (use_fp8 && w->tuning.scale_mode == 1) {
-            if (int rc = ensure_scale_stage(w, (size_t)R * max_tokens * (hidden / 128))) return rc;
-            stage = w->d_scale_stage;
+        if (!static_scratch) {
+            auto& ld = w->last;
+            ld.valid = true;
+            ld.hidden = hidden; ld.num_topk = num_topk; ld.max_tokens = max_tokens; ld.num_experts = num_experts;
+            ld.topk_idx.assign(topk_idx, topk_idx + R);
+            ld.recv_x.assign(recv_x, recv_x + R);
+            ld.src_info.assign(src_info, src_info + R);
+            ld.layout_range.assign(layout_range, layout_range + R);
+            ld.num_tokens.assign(num_tokens, num_tokens + R);
+            ld.plan = d.plan;
+            ld.captured = cap.active;
+            ld.capture_id = cap.id;
+            if (cap.active) w->dispatch_captured = true;
         }
+    }
+    if ((phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0)
         MC_HIP(launch_pack(d_tbl, sc, src, stage, d, use_fp8 != 0, w->tuning,
                            (phases & MC_EP_PHASE_DATA) != 0, (phases & MC_EP_PHASE_FINISH) != 0, stream));
-    }
     return MC_EP_OK;
 }
 
@@ -728,6 +776,14 @@ int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
     auto w = std::make_unique<mc_ep_world>();
     w->R = num_ranks;
     MC_HIP(hipGetDevice(&w->device));
+    // the device's copy of the static scratch array: its address is asked for once per device, here,
+    // with that device current; host code uses the pointer, never the array's name
+    if (w->device >= 0 && w->device < kMaxDevices && g_scratch_ptr[w->device] == nullptr) {
+        void* ptr = nullptr;
+        MC_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        MC_ASSERT(ptr != nullptr);
+        g_scratch_ptr[w->device] = (unsigned char*)ptr;
+    }
     MC_HIP(hipStreamCreateWithFlags(&w->comm_stream, hipStreamNonBlocking));
     for (int i = 0; i < 3; ++i) {
         const int fields[3] = {(int)DF_COUNT, (int)CF_COUNT, (int)XF_COUNT};
@@ -799,6 +855,18 @@ int mc_ep_world_dispatch(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_
     return world_dispatch_impl(w, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, max_tokens, num_experts,
                                use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
                                layout_range_ptrs, phases, (hipStream_t)stream_ptr);
+}
+
+int mc_ep_world_dispatch_noalloc(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_t* topk_idx_ptrs,
+                                 const int32_t* num_tokens, int hidden, int num_topk, int max_tokens,
+                                 int num_experts, int use_fp8, const uint64_t* recv_x_ptrs,
+                                 const uint64_t* recv_scales_ptrs, const uint64_t* recv_count_ptrs,
+                                 const uint64_t* src_info_ptrs, const uint64_t* layout_range_ptrs,
+                                 uint64_t stream_ptr) {
+    MC_ASSERT(w != nullptr);
+    return world_dispatch_impl(w, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, max_tokens, num_experts,
+                               use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
+                               layout_range_ptrs, MC_EP_PHASE_ALL, (hipStream_t)stream_ptr, true);
 }
 
 int mc_ep_world_combine(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_t* topk_idx_ptrs,

@@ -75,6 +75,18 @@ class World:
                 _lib.check(rc)
         return call
 
+    def dispatch_noalloc(self, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
+                         num_experts, use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
+                         layout_range_ptrs, stream_ptr: int) -> None:
+        """`dispatch` without any device allocation: its scratch is the library's static device array
+        (16 MiB per GPU, shared by every call on that GPU); larger shapes raise."""
+        u = _lib.u64_array
+        _lib.check(_lib.lib().mc_ep_world_dispatch_noalloc(
+            self._h, u(x_ptrs), u(topk_idx_ptrs), _lib.i32_array(num_tokens), hidden, num_topk,
+            num_max_dispatch_tokens_per_rank, num_experts, int(bool(use_fp8)), u(recv_x_ptrs),
+            u(recv_scales_ptrs) if recv_scales_ptrs is not None else None, u(recv_count_ptrs), u(src_info_ptrs),
+            u(layout_range_ptrs), stream_ptr))
+
     def prepare_combine(self, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
                         active_ranks_ptrs, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
                         num_experts, combined_x_ptrs):

@@ -77,10 +77,20 @@ class WorldHarness:
         return int(s.cuda_stream)
 
     def dispatch(self, phases: int = _lib.PHASE_ALL, stream: Optional[torch.cuda.Stream] = None,
-                 present: Optional[Sequence[int]] = None) -> None:
-        """present[r] == 0 makes rank r silent: it neither sends nor receives."""
+                 present: Optional[Sequence[int]] = None, noalloc: bool = False) -> None:
+        """present[r] == 0 makes rank r silent: it neither sends nor receives.  noalloc: through the
+        allocation-free entry point (all phases)."""
         c = self.cfg
         R = c.num_ranks
+        if noalloc:
+            nt = [n if (present is None or present[r]) else 0 for r, n in enumerate(self.num_tokens)]
+            self.world.dispatch_noalloc(
+                self._ptrs(self.x, R), self._ptrs(self.topk_idx, R), nt, c.hidden, c.num_topk, c.max_tokens,
+                c.num_experts, c.use_fp8, self._ptrs(self.recv_x, R, present),
+                self._ptrs(self.recv_scales_phys, R, present) if c.use_fp8 else None,
+                self._ptrs(self.recv_count, R, present), self._ptrs(self.src_info, R, present),
+                self._ptrs(self.layout_range, R, present), self._stream(stream))
+            return
         key = ("dispatch", None if present is None else tuple(present), self.x.data_ptr(), self.recv_x.data_ptr())
         call = self._prepared.get(key)
         if call is None:
