@@ -65,10 +65,13 @@ int mc_ep_world_create(int num_ranks, mc_ep_world_t** out);
 int mc_ep_world_destroy(mc_ep_world_t* world);
 int mc_ep_world_num_ranks(const mc_ep_world_t* world);
 
-/* A silent rank never calls dispatch/combine again (the reference's failed
+/* A silent rank stops calling dispatch/combine (the reference's failed
  * process, mooncake-ep/tests/test_ep_grid.py:121-158); collectives complete
  * without it.  Forces from the host what the reference detects by timeout
- * (mooncake_ep_kernel.cu:417-429, :688-698). */
+ * (mooncake_ep_kernel.cu:417-429, :688-698).  silent == 0 brings the rank back
+ * (the reference's restarted process, Buffer.update_ep_member,
+ * mooncake_ep_buffer.py:306-307): its next call joins the first round that no
+ * rank has opened yet. */
 int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
 
 /* Tuning knobs for measurement sweeps ("pack_variant", "pack_waves",
@@ -236,6 +239,14 @@ int mc_ep_buffer_combine(mc_ep_buffer_t* buffer, uint64_t x_ptr, uint64_t topk_i
                          uint64_t combined_x_ptr, int async, int return_recv_hook, uint64_t compute_stream_ptr,
                          mc_ep_event_t** event_out, mc_ep_hook_t** hook_out);
 
+/* How many of this rank's dispatch / combine calls still have kernels to be
+ * enqueued: their round waits for other live ranks, or (dispatch) for the
+ * receive hook that enqueues its second part.  The caller keeps the tensors of
+ * that many most recent calls of each kind alive; the reference's callers have
+ * no such duty because every process enqueues its own kernels inside the call
+ * (mooncake_ep_buffer.cpp:296-316). */
+int mc_ep_buffer_pending_calls(const mc_ep_buffer_t* buffer, int* dispatch_pending, int* combine_pending);
+
 /* ---- EventHandle (mooncake_ep_event.h:9-42) and the recv hook ----------- */
 
 /* EventHandle(stream_ptr): an event recorded on that stream now. */
@@ -244,8 +255,15 @@ int mc_ep_event_current_stream_wait(mc_ep_event_t* event, uint64_t stream_ptr);
 int mc_ep_event_synchronize(mc_ep_event_t* event);
 int mc_ep_event_destroy(mc_ep_event_t* event);
 
-/* The closure returned for return_recv_hook (mooncake_ep_buffer.cpp:330-335):
- * after it returns, work queued on the rank's compute stream sees the outputs. */
+/* The closure returned for return_recv_hook (mooncake_ep_buffer.cpp:303-305,
+ * :330-335).  A round whose callers all asked for a hook is launched in two
+ * parts, as the reference splits SEND and RECV: the call that completes the
+ * round enqueues MC_EP_PHASE_LAYOUT | MC_EP_PHASE_DATA, the first hook called
+ * enqueues MC_EP_PHASE_FINISH (an fp8 dispatch's scales; nothing for bf16 and
+ * for combine), and each hook makes its rank's compute stream wait for the
+ * round.  After it returns, work queued on that stream sees the outputs.  The
+ * next dispatch of the world enqueues a second part that no hook has asked for
+ * yet.  The hook must not outlive its world. */
 int mc_ep_hook_call(mc_ep_hook_t* hook);
 int mc_ep_hook_destroy(mc_ep_hook_t* hook);
 

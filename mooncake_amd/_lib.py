@@ -64,6 +64,7 @@ SIGNATURES = {
                                                POINTER(LegacyPerfResult)]),
     "mc_ep_buffer_create": (c_int, [c_void_p, c_int, c_int64, c_int, _VPP]),
     "mc_ep_buffer_destroy": (c_int, [c_void_p]),
+    "mc_ep_buffer_pending_calls": (c_int, [c_void_p, POINTER(c_int), POINTER(c_int)]),
     "mc_ep_buffer_ibgda_disabled": (c_int, [c_void_p]),
     "mc_ep_buffer_p2p_enabled": (c_int, [c_void_p]),
     "mc_ep_buffer_use_fast_path": (c_int, [c_void_p]),

@@ -83,7 +83,6 @@ struct RoutingScratch {
     int32_t* selpos;     // [R * max_tokens * K]  position inside (unit, expert); -1: no valid expert
     int32_t* counts;     // [E]     rows per expert (0 for experts of ranks that take no part)
     int32_t* row_src;    // [E, R * max_tokens]  packed row -> source token slot (rank * max_tokens + token)
-    uint32_t* ticket;    // [1]     blocks of the count kernel that have finished
 };
 
 // One resolved source row of combine's general path (a handle that is not the

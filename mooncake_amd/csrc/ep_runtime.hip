@@ -11,6 +11,7 @@
 #include <cstdio>
 #include <cstring>
 #include <deque>
+#include <functional>
 #include <memory>
 #include <string>
 #include <vector>
@@ -59,6 +60,12 @@ struct Round {
     bool launched = false;
     std::string failure;          // why the round's launch failed, if it did
     hipEvent_t done = nullptr;
+    // A round whose callers all asked for a receive hook is launched in two parts, like the
+    // reference's SEND / RECV phases (mooncake_ep_buffer.cpp:303-305, :330-335): the call that
+    // completes it enqueues the layout and data kernels, the first hook that is called enqueues the
+    // rest (`finish`) and records `done`; every hook then makes its rank's stream wait for `done`.
+    std::function<int()> finish;
+    hipStream_t launch_stream = nullptr;
     ~Round() {
         if (done) (void)hipEventDestroy(done);
     }
@@ -93,6 +100,12 @@ struct mc_ep_world {
     int device = 0;
     int R = 0;
     hipStream_t comm_stream = nullptr;
+    // Launch sequences of one world share its rank tables, routing state, routes and staged scales,
+    // so they are serialised: a sequence that runs on another stream than the one before it first
+    // waits for what that stream holds (order_begin).
+    hipEvent_t ordered = nullptr;
+    hipStream_t ordered_stream = nullptr;                // where the world's last eager sequence ran
+    bool ordered_valid = false;
     uint64_t* d_tbl[3] = {nullptr, nullptr, nullptr};   // dispatch, combine, consumer pointer tables
     std::vector<uint64_t> tbl_cache[3];                  // what the device tables hold
     // Calls recorded into a HIP graph get tables of their own (a replay must not depend on what later
@@ -113,8 +126,6 @@ struct mc_ep_world {
     size_t row_src_cap = 0;
     int32_t* d_counts = nullptr;
     size_t counts_cap = 0;
-    uint32_t* d_ticket = nullptr;
-    size_t ticket_cap = 0;
     uint32_t* d_chunk_map = nullptr;     // work list of the cast-back kernel, 4 words per entry
     size_t chunk_map_cap = 0;
     // what the last dispatch was called with, so that a combine given that
@@ -125,6 +136,7 @@ struct mc_ep_world {
         std::vector<uint64_t> topk_idx, recv_x, src_info, layout_range;
         std::vector<int32_t> num_tokens;
         UnitPlan plan;                            // how its routing state is laid out
+        bool data_done = false;                   // its pack phase has been launched too (and did not fail)
         bool captured = false;                    // recorded into a graph, and which capture
         unsigned long long capture_id = 0;
     } last;
@@ -134,6 +146,7 @@ struct mc_ep_world {
     float* d_scale_stage = nullptr;               // fp8 scales of each token before transposition
     size_t scale_stage_cap = 0;                   // capacity in floats
     void* d_zero_row = nullptr;
+    std::vector<void*> retired;                   // outgrown scratch, freed with the world
     Tuning tuning;
     std::vector<char> silent;
     // per-rank collective bookkeeping
@@ -141,6 +154,7 @@ struct mc_ep_world {
     std::deque<PendingRound<CombinePost>> combine_rounds;
     std::vector<long long> dispatch_calls, combine_calls;   // calls made per rank
     long long dispatch_base = 0, combine_base = 0;          // index of the front round
+    std::shared_ptr<Round> unfinished;                      // the dispatch round whose second part no hook has enqueued yet
 
     mc_ep_world() = default;
     mc_ep_world(const mc_ep_world&) = delete;
@@ -151,11 +165,13 @@ struct mc_ep_world {
         const bool switched = hipGetDevice(&prev) == hipSuccess && prev != device && hipSetDevice(device) == hipSuccess;
         (void)hipDeviceSynchronize();
         void* owned[] = {d_tbl[0], d_tbl[1], d_tbl[2], d_captured_tbl[0], d_captured_tbl[1], d_captured_tbl[2],
-                         d_ucount, d_ucount_t, d_ubegin, d_selpos, d_row_src, d_counts, d_ticket, d_chunk_map, d_routes,
+                         d_ucount, d_ucount_t, d_ubegin, d_selpos, d_row_src, d_counts, d_chunk_map, d_routes,
                          d_scale_stage, d_zero_row};
         for (void* p : owned)
             if (p) (void)hipFree(p);
+        for (void* p : retired) (void)hipFree(p);
         if (comm_stream) (void)hipStreamDestroy(comm_stream);
+        if (ordered) (void)hipEventDestroy(ordered);
         if (switched) (void)hipSetDevice(prev);
     }
 };
@@ -173,6 +189,7 @@ struct mc_ep_event {
 };
 
 struct mc_ep_hook {
+    mc_ep_world* world = nullptr;
     std::shared_ptr<Round> round;
     hipStream_t stream = nullptr;
 };
@@ -228,49 +245,45 @@ struct RecordingScope {
                         "the same call once outside the capture first");                                        \
     } while (0)
 
-int ensure_routes(mc_ep_world* w, size_t selections) {
-    if (selections <= w->route_cap) return MC_EP_OK;
-    MC_NO_GROWTH_WHILE_RECORDING();
-    // grows only; the old table may still be read by queued kernels
-    MC_HIP(hipDeviceSynchronize());
-    if (w->d_routes) MC_HIP(hipFree(w->d_routes));
-    w->d_routes = nullptr;
-    w->route_cap = 0;
-    const size_t cap = selections + selections / 2 + 1024;
-    MC_HIP(hipMalloc((void**)&w->d_routes, cap * sizeof(CombineRoute)));
-    // stamps start at 1, so a zeroed table holds no valid route
-    MC_HIP(hipMemset(w->d_routes, 0, cap * sizeof(CombineRoute)));
-    w->stamp = 0;
-    w->route_cap = cap;
-    return MC_EP_OK;
-}
-
+// Scratch grows by replacement.  The outgrown allocation is kept until the world is destroyed
+// (`retired`): kernels already queued, and graphs instantiated while it was current, hold its address
+// in their arguments and go on using it - a graph's calls are self-contained (a recorded combine
+// reuses only a dispatch of its own capture), so they stay right on the old memory.  Sizes grow
+// geometrically, so the retired total stays below twice the live one.
 template <typename T>
-int ensure_scratch(T** ptr, size_t* cap, size_t count) {
+int grow_scratch(mc_ep_world* w, T** ptr, size_t* cap, size_t count, bool zero) {
     if (count <= *cap) return MC_EP_OK;
     MC_NO_GROWTH_WHILE_RECORDING();
-    MC_HIP(hipDeviceSynchronize());
-    if (*ptr) MC_HIP(hipFree(*ptr));
-    *ptr = nullptr;
-    *cap = 0;
     const size_t grown = count + count / 2 + 1024;
-    MC_HIP(hipMalloc((void**)ptr, grown * sizeof(T)));
-    MC_HIP(hipMemset(*ptr, 0, grown * sizeof(T)));
+    T* fresh = nullptr;
+    MC_HIP(hipMalloc((void**)&fresh, grown * sizeof(T)));
+    if (zero) {
+        const hipError_t e = hipMemset(fresh, 0, grown * sizeof(T));
+        // the fill must have landed before a kernel on any stream reads the new memory
+        const hipError_t e2 = e == hipSuccess ? hipStreamSynchronize(nullptr) : e;
+        if (e2 != hipSuccess) {
+            (void)hipFree(fresh);
+            MC_HIP(e2);
+        }
+    }
+    if (*ptr) w->retired.push_back(*ptr);
+    *ptr = fresh;
     *cap = grown;
     return MC_EP_OK;
 }
 
+// stamps start at 1 and are never reset, so a zeroed route table holds no valid route
+int ensure_routes(mc_ep_world* w, size_t selections) {
+    return grow_scratch(w, &w->d_routes, &w->route_cap, selections, true);
+}
+
+template <typename T>
+int ensure_scratch(mc_ep_world* w, T** ptr, size_t* cap, size_t count) {
+    return grow_scratch(w, ptr, cap, count, true);
+}
+
 int ensure_scale_stage(mc_ep_world* w, size_t floats) {
-    if (floats <= w->scale_stage_cap) return MC_EP_OK;
-    MC_NO_GROWTH_WHILE_RECORDING();
-    MC_HIP(hipDeviceSynchronize());
-    if (w->d_scale_stage) MC_HIP(hipFree(w->d_scale_stage));
-    w->d_scale_stage = nullptr;
-    w->scale_stage_cap = 0;
-    const size_t cap = floats + floats / 2 + 1024;
-    MC_HIP(hipMalloc((void**)&w->d_scale_stage, cap * sizeof(float)));
-    w->scale_stage_cap = cap;
-    return MC_EP_OK;
+    return grow_scratch(w, &w->d_scale_stage, &w->scale_stage_cap, floats, false);
 }
 
 // Puts the call's rank table on the device and returns where.  Eager calls share one table per kind,
@@ -340,7 +353,39 @@ int uniform_tokens(const int32_t* n, int R, bool enabled) {
 }
 
 RoutingScratch routing_scratch(const mc_ep_world* w) {
-    return RoutingScratch{w->d_ucount, w->d_ucount_t, w->d_ubegin, w->d_selpos, w->d_counts, w->d_row_src, w->d_ticket};
+    return RoutingScratch{w->d_ucount, w->d_ucount_t, w->d_ubegin, w->d_selpos, w->d_counts, w->d_row_src};
+}
+
+// Enqueues what is left of a round that was launched in two parts (see Round::finish).
+int finish_round(mc_ep_world* w, Round* round) {
+    if (!round->finish) return MC_EP_OK;
+    const std::function<int()> rest = std::move(round->finish);
+    round->finish = nullptr;
+    if (w->unfinished.get() == round) w->unfinished.reset();
+    const int e = rest();
+    if (e) round->failure = g_last_error;
+    return e;
+}
+
+// Serialisation of a world's launch sequences across streams (see mc_ep_world::ordered).  Nothing is
+// recorded while the world stays on one stream (an event per call costs 3-4 us of device time each);
+// when a sequence arrives on another stream, the event is recorded on the previous stream then - it
+// covers everything queued there so far, the world's earlier sequences included - and the new stream
+// waits for it.  Calls being recorded into a graph take no part: a graph's order is its capturing
+// stream's, and a stream that is capturing cannot be asked for an event of eager work.
+int order_begin(mc_ep_world* w, hipStream_t stream, const Capture& cap) {
+    if (cap.active) return MC_EP_OK;
+    if (w->ordered_valid && w->ordered_stream != stream) {
+        Capture prev;
+        if (int rc = capture_of(w->ordered_stream, &prev)) return rc;
+        if (!prev.active) {
+            MC_HIP(hipEventRecord(w->ordered, w->ordered_stream));
+            MC_HIP(hipStreamWaitEvent(stream, w->ordered, 0));
+        }
+    }
+    w->ordered_stream = stream;
+    w->ordered_valid = true;
+    return MC_EP_OK;
 }
 
 int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_idx, const int32_t* num_tokens,
@@ -378,6 +423,10 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         if (num_tokens[r] > tgrid) tgrid = num_tokens[r];
     }
     DeviceGuard guard(w->device);
+    // a new dispatch overwrites the staged scales and the routing state: the second part of a round
+    // that still waits for its hook has to be enqueued first
+    if (!static_scratch && (phases & MC_EP_PHASE_LAYOUT) && w->unfinished)
+        if (int rc = finish_round(w, w->unfinished.get())) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
     plan_units(d, w->tuning);
     // the count kernel keeps per-wave counts and prefixes of every expert in LDS
@@ -421,12 +470,13 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     } else {
         if (int rc = capture_of(stream, &cap)) return rc;
         RecordingScope recording(cap.active);
-        if (int rc = ensure_scratch(&w->d_ucount, &w->ucount_cap, UE)) return rc;
-        if (int rc = ensure_scratch(&w->d_ubegin, &w->ubegin_cap, UE)) return rc;
-        if (int rc = ensure_scratch(&w->d_ucount_t, &w->ucount_t_cap, (size_t)num_experts * kMaxSummedUnits)) return rc;
-        if (int rc = ensure_scratch(&w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
-        if (int rc = ensure_scratch(&w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
-        if (int rc = ensure_scratch(&w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
+        if (int rc = order_begin(w, stream, cap)) return rc;
+        if (int rc = ensure_scratch(w, &w->d_ucount, &w->ucount_cap, UE)) return rc;
+        if (int rc = ensure_scratch(w, &w->d_ubegin, &w->ubegin_cap, UE)) return rc;
+        if (int rc = ensure_scratch(w, &w->d_ucount_t, &w->ucount_t_cap, (size_t)num_experts * kMaxSummedUnits)) return rc;
+        if (int rc = ensure_scratch(w, &w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
+        if (int rc = ensure_scratch(w, &w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
+        if (int rc = ensure_scratch(w, &w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
         if (stage_floats > 0 && (phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
             if (int rc = ensure_scale_stage(w, stage_floats)) return rc;
             stage = w->d_scale_stage;
@@ -455,12 +505,16 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
             ld.plan = d.plan;
             ld.captured = cap.active;
             ld.capture_id = cap.id;
+            ld.data_done = false;
             if (cap.active) w->dispatch_captured = true;
         }
     }
     if ((phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0)
         MC_HIP(launch_pack(d_tbl, sc, src, stage, d, use_fp8 != 0, w->tuning,
                            (phases & MC_EP_PHASE_DATA) != 0, (phases & MC_EP_PHASE_FINISH) != 0, stream));
+    // under the carried plan the pack launch also produces ubegin and the counts: only now is the
+    // routing state complete for a combine to reuse
+    if (!static_scratch && (phases & MC_EP_PHASE_DATA)) w->last.data_done = true;
     return MC_EP_OK;
 }
 
@@ -497,6 +551,7 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     Capture cap;
     if (int rc = capture_of(stream, &cap)) return rc;
     RecordingScope recording(cap.active);
+    if (int rc = order_begin(w, stream, cap)) return rc;
     const uint64_t* d_tbl = nullptr;
     if (int rc = upload_table(w, 1, tbl, cap, stream, &d_tbl)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
@@ -508,7 +563,7 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     // the combine of its handle (mooncake_ep_kernel.cu:734 finds a token's rows
     // by its dispatch-time expert indices).
     const auto& ld = w->last;
-    bool direct = w->tuning.combine_direct != 0 && ld.valid && ld.hidden == hidden && ld.num_topk == num_topk &&
+    bool direct = w->tuning.combine_direct != 0 && ld.valid && ld.data_done && ld.hidden == hidden && ld.num_topk == num_topk &&
                   ld.max_tokens == max_tokens && ld.num_experts == num_experts;
     // "Last" is about the order on the device.  Graph replays run dispatches the host never sees, so: a
     // recorded combine trusts only a dispatch recorded in the same capture, and once a dispatch of this
@@ -649,11 +704,33 @@ int launch_dispatch_round(mc_ep_world* w, PendingRound<DispatchPost>& pr) {
     hipStream_t launch = pick_launch_stream(w, pr.posts, &shared);
     if (int e = fence_before(w, pr.posts, launch)) return e;
     if (int e = mark_silent_inactive(w, pr.posts, launch)) return e;
-    if (int e = world_dispatch_impl(w, x.data(), idx.data(), nt.data(), first->hidden, first->num_topk,
-                                    first->max_tokens, first->num_experts, first->use_fp8, rx.data(), rs.data(),
-                                    rc.data(), si.data(), lr.data(), MC_EP_PHASE_ALL, launch))
+    bool all_hook = true;
+    for (const auto& p : pr.posts)
+        if (p.present && !p.hook) all_hook = false;
+    // only an fp8 dispatch has a second part (the scales' move into their column-major layout)
+    const bool two_part = all_hook && first->use_fp8;
+    const int hidden = first->hidden, num_topk = first->num_topk, max_tokens = first->max_tokens,
+              num_experts = first->num_experts, use_fp8 = first->use_fp8;
+    if (int e = world_dispatch_impl(w, x.data(), idx.data(), nt.data(), hidden, num_topk, max_tokens, num_experts,
+                                    use_fp8, rx.data(), rs.data(), rc.data(), si.data(), lr.data(),
+                                    two_part ? (MC_EP_PHASE_LAYOUT | MC_EP_PHASE_DATA) : MC_EP_PHASE_ALL, launch))
         return e;
-    return fence_after(pr.posts, launch, pr.state.get());
+    Round* round = pr.state.get();
+    round->launch_stream = launch;
+    if (!two_part) return fence_after(pr.posts, launch, round);
+    MC_HIP(hipEventCreateWithFlags(&round->done, hipEventDisableTiming));
+    round->finish = [=]() -> int {
+        DeviceGuard g(w->device);
+        if (int e = world_dispatch_impl(w, x.data(), idx.data(), nt.data(), hidden, num_topk, max_tokens, num_experts,
+                                        use_fp8, rx.data(), rs.data(), rc.data(), si.data(), lr.data(),
+                                        MC_EP_PHASE_FINISH, launch))
+            return e;
+        MC_HIP(hipEventRecord(round->done, launch));
+        return MC_EP_OK;
+    };
+    w->unfinished = pr.state;
+    round->launched = true;
+    return MC_EP_OK;
 }
 
 int launch_combine_round(mc_ep_world* w, PendingRound<CombinePost>& pr) {
@@ -684,6 +761,7 @@ int launch_combine_round(mc_ep_world* w, PendingRound<CombinePost>& pr) {
                                    first->hidden, first->num_topk, first->max_tokens, first->num_experts,
                                    out.data(), MC_EP_PHASE_ALL, launch))
         return e;
+    pr.state->launch_stream = launch;
     return fence_after(pr.posts, launch, pr.state.get());
 }
 
@@ -717,16 +795,19 @@ int drain_combine(mc_ep_world* w) {
     return MC_EP_OK;
 }
 
+// The round a rank's call_index-th call belongs to (opened on demand), or null for a call index that
+// lies before the front round, which the callers turn into an assertion failure.
 template <typename Post>
-PendingRound<Post>& round_for_call(mc_ep_world* w, std::deque<PendingRound<Post>>& rounds, long long base,
+PendingRound<Post>* round_for_call(mc_ep_world* w, std::deque<PendingRound<Post>>& rounds, long long base,
                                    long long call_index) {
+    if (call_index < base) return nullptr;
     while ((long long)rounds.size() <= call_index - base) {
         PendingRound<Post> pr;
         pr.posts.resize(w->R);
         pr.state = std::make_shared<Round>();
         rounds.push_back(std::move(pr));
     }
-    return rounds[(size_t)(call_index - base)];
+    return &rounds[(size_t)(call_index - base)];
 }
 
 // What a waiter on a round that cannot complete is told: either the launch failed (the call that
@@ -785,6 +866,7 @@ int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
         g_scratch_ptr[w->device] = (unsigned char*)ptr;
     }
     MC_HIP(hipStreamCreateWithFlags(&w->comm_stream, hipStreamNonBlocking));
+    MC_HIP(hipEventCreateWithFlags(&w->ordered, hipEventDisableTiming));
     for (int i = 0; i < 3; ++i) {
         const int fields[3] = {(int)DF_COUNT, (int)CF_COUNT, (int)XF_COUNT};
         const size_t words = (size_t)fields[i] * num_ranks;
@@ -809,7 +891,16 @@ int mc_ep_world_num_ranks(const mc_ep_world_t* w) { return w ? w->R : 0; }
 
 int mc_ep_world_set_rank_silent(mc_ep_world_t* w, int rank, int silent) {
     MC_ASSERT(w != nullptr && rank >= 0 && rank < w->R);
+    const bool was_silent = w->silent[rank] != 0;
     w->silent[rank] = silent ? 1 : 0;
+    if (was_silent && !silent) {
+        // A rank that comes back (the reference's update_ep_member after a restart) has missed the
+        // rounds that completed without it and the ones its peers have already opened: its next call
+        // joins the first round nobody has opened yet.
+        w->dispatch_calls[rank] = w->dispatch_base + (long long)w->dispatch_rounds.size();
+        w->combine_calls[rank] = w->combine_base + (long long)w->combine_rounds.size();
+        return MC_EP_OK;
+    }
     // rounds that were only waiting for this rank can go now
     if (int e = drain_dispatch(w)) return e;
     return drain_combine(w);
@@ -907,6 +998,7 @@ int mc_ep_world_cast_back(mc_ep_world_t* w, const uint64_t* recv_x_ptrs, const u
     Capture cap;
     if (int rc = capture_of(stream, &cap)) return rc;
     RecordingScope recording(cap.active);
+    if (int rc = order_begin(w, stream, cap)) return rc;
     const uint64_t* d_tbl = nullptr;
     if (int rc = upload_table(w, 2, tbl, cap, stream, &d_tbl)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, max_tokens};
@@ -914,7 +1006,7 @@ int mc_ep_world_cast_back(mc_ep_world_t* w, const uint64_t* recv_x_ptrs, const u
     long long max_rows = (long long)num_experts * R * max_tokens;
     if (num_topk > 0 && (long long)R * max_tokens * num_topk < max_rows) max_rows = (long long)R * max_tokens * num_topk;
     const size_t map_words = (size_t)(cast_back_chunks(max_rows, num_experts) + 1) * 4;
-    if (int rc = ensure_scratch(&w->d_chunk_map, &w->chunk_map_cap, map_words)) return rc;
+    if (int rc = ensure_scratch(w, &w->d_chunk_map, &w->chunk_map_cap, map_words)) return rc;
     MC_HIP(launch_cast_back(d_tbl, w->d_chunk_map, (const float*)expert_factor_ptr, use_fp8, max_rows, d,
                             stream));
     return MC_EP_OK;
@@ -1024,6 +1116,19 @@ int mc_ep_buffer_destroy(mc_ep_buffer_t* b) {
     return MC_EP_OK;
 }
 
+int mc_ep_buffer_pending_calls(const mc_ep_buffer_t* b, int* dispatch_pending, int* combine_pending) {
+    MC_ASSERT(b != nullptr && dispatch_pending != nullptr && combine_pending != nullptr);
+    const mc_ep_world* w = b->world;
+    long long d = w->dispatch_calls[b->rank] - w->dispatch_base;
+    long long c = w->combine_calls[b->rank] - w->combine_base;
+    if (d < 0) d = 0;
+    if (c < 0) c = 0;
+    if (w->unfinished) d += 1;   // launched in part: its second part still reads the round's tensors
+    *dispatch_pending = (int)d;
+    *combine_pending = (int)c;
+    return MC_EP_OK;
+}
+
 int mc_ep_buffer_ibgda_disabled(const mc_ep_buffer_t*) { return 1; }
 int mc_ep_buffer_p2p_enabled(const mc_ep_buffer_t* b) { return b && b->p2p_enabled ? 1 : 0; }
 int mc_ep_buffer_use_fast_path(const mc_ep_buffer_t*) { return 1; }
@@ -1061,8 +1166,11 @@ int mc_ep_buffer_dispatch(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_p
     MC_ASSERT(num_topk <= kMaxTopK);
     MC_ASSERT(!w->silent[b->rank]);
 
-    const long long call = w->dispatch_calls[b->rank]++;
-    auto& pr = round_for_call(w, w->dispatch_rounds, w->dispatch_base, call);
+    const long long call = w->dispatch_calls[b->rank];
+    auto* prp = round_for_call(w, w->dispatch_rounds, w->dispatch_base, call);
+    MC_ASSERT(prp != nullptr);
+    w->dispatch_calls[b->rank] = call + 1;
+    auto& pr = *prp;
     DispatchPost& p = pr.posts[b->rank];
     p.present = true;
     p.x = x_ptr; p.topk_idx = topk_idx_ptr; p.active_ranks = active_ranks_ptr;
@@ -1082,6 +1190,7 @@ int mc_ep_buffer_dispatch(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_p
     }
     if (return_recv_hook) {
         auto* h = new mc_ep_hook();
+        h->world = w;
         h->round = state;
         h->stream = (hipStream_t)compute_stream_ptr;
         *hook_out = h;
@@ -1120,8 +1229,11 @@ int mc_ep_buffer_combine(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_pt
     MC_ASSERT(num_topk <= kMaxTopK);
     MC_ASSERT(!w->silent[b->rank]);
 
-    const long long call = w->combine_calls[b->rank]++;
-    auto& pr = round_for_call(w, w->combine_rounds, w->combine_base, call);
+    const long long call = w->combine_calls[b->rank];
+    auto* prp = round_for_call(w, w->combine_rounds, w->combine_base, call);
+    MC_ASSERT(prp != nullptr);
+    w->combine_calls[b->rank] = call + 1;
+    auto& pr = *prp;
     CombinePost& p = pr.posts[b->rank];
     p.present = true;
     p.x = x_ptr; p.topk_idx = topk_idx_ptr; p.topk_weights = topk_weights_ptr; p.src_info = src_info_ptr;
@@ -1140,6 +1252,7 @@ int mc_ep_buffer_combine(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_pt
     }
     if (return_recv_hook) {
         auto* h = new mc_ep_hook();
+        h->world = w;
         h->round = state;
         h->stream = (hipStream_t)compute_stream_ptr;
         *hook_out = h;
@@ -1188,7 +1301,12 @@ int mc_ep_event_destroy(mc_ep_event_t* ev) {
 int mc_ep_hook_call(mc_ep_hook_t* h) {
     MC_ASSERT(h != nullptr);
     if (!h->round || !h->round->launched) return round_not_ready(h->round.get());
-    MC_HIP(hipStreamWaitEvent(h->stream, h->round->done, 0));
+    // the first hook of a round launched in two parts enqueues the second part (the reference's
+    // RECV phase, mooncake_ep_buffer.cpp:330-335)
+    if (h->round->finish)
+        if (int e = finish_round(h->world, h->round.get())) return e;
+    if (!h->round->failure.empty()) return round_not_ready(h->round.get());
+    if (h->stream != h->round->launch_stream) MC_HIP(hipStreamWaitEvent(h->stream, h->round->done, 0));
     return MC_EP_OK;
 }
 

@@ -229,6 +229,12 @@ class Buffer:
         except Exception:
             pass
 
+    def pending_calls(self) -> Tuple[int, int]:
+        """(dispatch, combine) calls of this rank whose kernels are not all enqueued yet."""
+        d, c = ctypes.c_int(), ctypes.c_int()
+        _lib.check(_lib.lib().mc_ep_buffer_pending_calls(self._h, ctypes.byref(d), ctypes.byref(c)))
+        return d.value, c.value
+
     # --- transport introspection: one address space, no NIC ---------------
     def ibgda_disabled(self) -> bool:
         return bool(_lib.lib().mc_ep_buffer_ibgda_disabled(self._h))

@@ -81,12 +81,31 @@ class Buffer:
         self.runtime = ep.Buffer(self.rank, self.group_size, num_ep_buffer_bytes, disable_p2p, world=world)
         # there is no slow path here: the HIP kernels are the only implementation
         self._use_fallback = False
-        # a round is launched by its last rank's call, which comes before this
-        # rank's next call of the same kind: keeping the tensors of the last
-        # two dispatches and combines alive covers it (a longer history would
-        # pin gigabytes of packed buffers per rank)
-        self._keepalive = collections.deque(maxlen=4)
+        # A round's kernels are enqueued by the call of its last rank, with the raw addresses every
+        # rank posted: the tensors of a call stay referenced here until the runtime reports that the
+        # call's round has been enqueued (however far ahead of its peers this rank runs).
+        self._posted_dispatch = collections.deque()
+        self._posted_combine = collections.deque()
         self.connect()
+
+    def _retain(self, posted: collections.deque, tensors: tuple, kind: int) -> None:
+        posted.append(tensors)
+        pending = self.runtime.pending_calls()[kind]
+        while len(posted) > pending:
+            posted.popleft()
+
+    @staticmethod
+    def _hook_keeping(hook: Optional[Callable], tensors: tuple) -> Optional[Callable]:
+        """The receive hook, holding the call's tensors until it has run: in hook mode nothing else
+        orders the caller's later work on those tensors after the round's kernels."""
+        if hook is None:
+            return None
+        kept = [tensors]
+
+        def call() -> None:
+            hook()
+            kept.clear()
+        return call
 
     def connect(self, is_update: bool = False) -> None:
         """Peer exchange of the reference (:185-304; is_update re-runs it for a changed membership, :306-307)
@@ -155,9 +174,10 @@ class Buffer:
                   num_experts)
         tensors_to_record = (x, topk_idx, active_ranks, packed_recv_x, packed_recv_x_scales, packed_recv_count,
                              packed_recv_src_info, packed_recv_layout_range)
-        self._keepalive.append(tensors_to_record)
+        self._retain(self._posted_dispatch, tensors_to_record, 0)
         return ((packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x, packed_recv_count, handle,
-                EventOverlap(event, tensors_to_record if async_finish else None), hook)
+                EventOverlap(event, tensors_to_record if async_finish else None),
+                self._hook_keeping(hook, tensors_to_record))
 
     # noinspection PyTypeChecker
     def combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
@@ -207,8 +227,9 @@ class Buffer:
             topk_weights.size(1), num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy,
             combined_x.data_ptr(), async_finish, return_recv_hook, _native_current_stream_ptr())
         tensors_to_record = (x, topk_idx, topk_weights, active_ranks, src_info, layout_range, combined_x)
-        self._keepalive.append(tensors_to_record)
-        return combined_x, EventOverlap(event, tensors_to_record if async_finish else None), hook
+        self._retain(self._posted_combine, tensors_to_record, 1)
+        return (combined_x, EventOverlap(event, tensors_to_record if async_finish else None),
+                self._hook_keeping(hook, tensors_to_record))
 
     def get_next_combine_buffer(self, handle: object):
         raise NotImplementedError(_ZERO_COPY_COMBINE_UNSUPPORTED)
