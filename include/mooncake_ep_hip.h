@@ -155,6 +155,23 @@ int mc_ep_world_cast_back(mc_ep_world_t* world, const uint64_t* packed_recv_x_pt
                           uint64_t expert_factor_ptr, const uint64_t* out_ptrs, int hidden, int num_topk,
                           int num_max_dispatch_tokens_per_rank, int num_experts, uint64_t stream_ptr);
 
+/* Combine fused with that consumer: what mc_ep_world_cast_back (with the same
+ * packed_recv_x / scales / expert_factor arguments) followed by
+ * mc_ep_world_combine on its output computes, bit for bit, without writing
+ * and re-reading the bf16 rows in between: every source row becomes
+ * bf16(bf16(f32(fp8) * scale) * factor[expert]) in registers (the grid test's
+ * mock expert, mooncake-ep/tests/test_ep_grid.py:160-173, between dispatch and
+ * combine) and enters the fp32 sum of mooncake_ep_kernel.cu:711-753.
+ * packed_recv_x_scales_ptrs == NULL: bf16 payload; expert_factor_ptr == 0: no
+ * factor.  The other arguments are mc_ep_world_combine's. */
+int mc_ep_world_combine_packed(mc_ep_world_t* world, const uint64_t* packed_recv_x_ptrs,
+                               const uint64_t* packed_recv_x_scales_ptrs, uint64_t expert_factor_ptr,
+                               const uint64_t* topk_idx_ptrs, const uint64_t* topk_weights_ptrs,
+                               const uint64_t* src_info_ptrs, const uint64_t* layout_range_ptrs,
+                               const uint64_t* active_ranks_ptrs, const int32_t* num_combined_tokens, int hidden,
+                               int num_topk, int num_max_dispatch_tokens_per_rank, int num_experts,
+                               const uint64_t* combined_x_ptrs, int phases, uint64_t stream_ptr);
+
 /* ---- the native benchmark loop ------------------------------------------ */
 
 /* _benchmark_legacy_buffer (bound in mooncake-ep/src/ep_py.cpp:12,26; the loop

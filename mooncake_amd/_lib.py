@@ -58,6 +58,8 @@ SIGNATURES = {
                                              _U64P, _U64P, _U64P, _U64P, _U64P, c_uint64]),
     "mc_ep_world_combine": (c_int, [c_void_p, _U64P, _U64P, _U64P, _U64P, _U64P, _U64P, _I32P, c_int, c_int,
                                     c_int, c_int, _U64P, c_int, c_uint64]),
+    "mc_ep_world_combine_packed": (c_int, [c_void_p, _U64P, _U64P, c_uint64, _U64P, _U64P, _U64P, _U64P, _U64P, _I32P,
+                                           c_int, c_int, c_int, c_int, _U64P, c_int, c_uint64]),
     "mc_ep_world_cast_back": (c_int, [c_void_p, _U64P, _U64P, _U64P, c_uint64, _U64P, c_int, c_int, c_int, c_int,
                                       c_uint64]),
     "mc_ep_world_legacy_buffer_perf": (c_int, [c_void_p, POINTER(LegacyPerfTensors), POINTER(LegacyPerfConfig),

@@ -32,6 +32,7 @@ enum CombineField : int {
     CF_ACTIVE,         // const int32* [R]  the rank's own view of live ranks
     CF_OUT,            // bf16*        [T_r, H]
     CF_NUM_TOKENS,     // T_r as an integer (0: rank combines nothing)
+    CF_SCALES,         // const float* [L, H/128, R*max]: scales of an fp8 payload in CF_X (packed combine only)
     CF_COUNT
 };
 
@@ -89,7 +90,7 @@ struct RoutingScratch {
 // one the last dispatch produced): valid for the launch whose stamp it carries,
 // so selections that no routing thread visits need no clearing pass.
 struct CombineRoute {       // 16 bytes
-    uint64_t src;           // byte address of the expert-output row
+    uint64_t src;           // byte address of the expert-output row; packed combine: (expert << 32) | row in its block
     float weight;
     uint32_t stamp;
 };
@@ -126,11 +127,11 @@ struct Dims {
 
 // Tuning knobs, settable at run time for measurement sweeps.
 struct Tuning {
-    int pack_variant = 0;      // 0: 32 B/lane loads, 16 B stores; 1: two coalesced 16 B loads, 8 B stores
     int pack_waves = 4;        // waves per block in the pack kernel
-    int pack_nt = -1;          // bit 0: streaming (nontemporal) loads, bit 1: streaming stores; -1: by top-k
+    int pack_nt = -1;          // 1: streaming (nontemporal) loads, 0: ordinary loads; -1: by top-k
     int uniform = 1;           // take per-rank addresses from kernel arguments when tensors are evenly spaced
-    int scale_mode = 1;        // 0: scatter scales from the pack kernel; 1: staged + transposing pass
+    int fp8_arith = 0;         // fp8 scale arithmetic: 0 = the reference's PyTorch statement as CPU PyTorch runs it,
+                               // 1 = the reference kernel's own (see pack_fp8_kernel)
     int combine_direct = 1;    // reuse the last dispatch's routing state when combine gets that dispatch's handle
     int combine_chunks = 0;    // 16-byte chunks per lane in the combine kernel (1 or 2); 0: by top-k
     int combine_waves = 4;     // waves per block in the combine kernel
@@ -148,12 +149,19 @@ hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const D
 hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, float* scale_stage,
                        const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
                        hipStream_t stream);
-hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, const Dims& d,
+// packed: routes carry (expert, row) instead of a row address
+hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, bool packed, const Dims& d,
                           const Tuning& t, hipStream_t stream);
 // direct: rows come from the last dispatch's routing state (sc); otherwise from d_routes
 hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp, const RoutingScratch& sc,
                          bool direct, const CombineSource& src, const void* d_zero_row, const Dims& d, const Tuning& t,
                          hipStream_t stream);
+// Combine straight from the packed layout: CF_X holds dispatch's payload (fp8 with CF_SCALES, or bf16), every
+// row is turned into what the consumer kernel would have made of it (times factor[expert] when d_factor is
+// given) on its way into the weighted sum.
+hipError_t launch_reduce_packed(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp,
+                                const RoutingScratch& sc, bool direct, const CombineSource& src, const void* d_zero_row,
+                                const float* d_factor, bool use_fp8, const Dims& d, const Tuning& t, hipStream_t stream);
 // packed rows below packed_recv_count -> bf16 rows times factor[expert]; max_rows bounds the world's valid rows
 // d_chunk_map: 16 bytes x (cast_back_chunks(max_rows, E) + 1) of scratch for the kernel's work list
 long long cast_back_chunks(long long max_rows, int num_experts);

@@ -15,8 +15,12 @@
 //                   token ascending, as the reference's PyTorch statement has
 //                   it (mooncake-wheel/mooncake/mooncake_ep_buffer.py:787-817).
 //   pack_kernel     one read of each token row, optional bf16 -> fp8 e4m3
-//                   quantisation with per-128 amax / 448 scales
-//                   (mooncake_ep_kernel.cu:183-186, :233-264), K row stores
+//                   quantisation with per-128 amax / 448 scales (the contract
+//                   of mooncake_ep_kernel.cu:183-186, :233-264; the scale
+//                   arithmetic follows, by default, the reference's PyTorch
+//                   statement of it, mooncake_ep_buffer.py:693-703, and the
+//                   kernel's own on request - they differ in the last bit of
+//                   the scale for about a quarter of all groups), K row stores
 //                   straight into [local expert, R*max, hidden]
 //                   (the reference needs two hops, :273-306 then :442-466);
 //                   scale_transpose_kernel then moves the fp8 scales into
@@ -53,6 +57,19 @@ __device__ __forceinline__ float group_max(float v) {
     v = fmaxf(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
     v = fmaxf(v, dpp_move<0x141>(v));   // row_half_mirror
     if (GROUP == 16) v = fmaxf(v, dpp_move<0x140>(v));   // row_mirror
+    return v;
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave (all of them active), in the DPP data path: shifts
+// by 1, 2, 4, 8 inside each row of 16 lanes (zeros shifted in), then lane 15 of rows 0 and 2 added to
+// rows 1 and 3, then lane 31 added to rows 2 and 3.
+__device__ __forceinline__ int wave_scan_inclusive(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, true);    // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, true);    // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, true);    // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, true);    // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);   // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);   // row_bcast:31 into rows 2 and 3
     return v;
 }
 
@@ -194,18 +211,13 @@ __device__ __forceinline__ void prefix_expert(const uint64_t* __restrict__ tbl, 
     for (int u0 = 0; u0 < U; u0 += 64) {
         const int u = u0 + lane;
         const int c = (u < U) ? sc.ucount[(int64_t)u * E + ee] : 0;
-        int incl = c;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const int up = __shfl_up(incl, d);
-            if (lane >= d) incl += up;
-        }
+        const int incl = wave_scan_inclusive(c);
         if (u < U) {
             const int excl = carry + incl - c;
             sc.ubegin[(int64_t)u * E + ee] = excl;
             pre[u] = excl;
         }
-        carry += __shfl(incl, 63);
+        carry += __builtin_amdgcn_readlane(incl, 63);
     }
     if (lane == 0) pre[U] = carry;
     // the same wave wrote pre[] and reads it below: a wave's LDS accesses complete in order
@@ -334,7 +346,6 @@ constexpr int kMaxPackWaves = 8;     // waves per block the launcher may choose
 // K times.
 struct PackDest {
     uint64_t row;     // byte address of the destination row, 0 = no store
-    uint64_t scale;   // byte address of scales[le][0][slot] (fp8)
 };
 
 // The lanes that work on selection k (lane k, or a group of sel_stride() lanes under the summed
@@ -352,15 +363,13 @@ __device__ __forceinline__ PackDest pack_destination(const uint64_t* __restrict_
     // the dependent gathers, side by side; the table's come first because the summed begin waits for
     // its own loads inside, and whatever is issued after that wait is a round trip later
     const uint64_t base = tbl[DF_RECV_X * R + k.q];
-    const uint64_t sbase = FP8 ? tbl[DF_RECV_SCALES * R + k.q] : 0;
     const uint64_t info = (slab == 0) ? tbl[DF_SRC_INFO * R + k.q] : 0;
     const int ub = up.summed ? summed_begin(sc, k, up, r, t, K, j, stride) : sc.ubegin[(int64_t)k.unit * E + k.e];
     const SelRow s = selection_row(k, ub, R, max_tokens);
-    PackDest d = {0, 0};
+    PackDest d = {0};
     if (s.ok && base != 0) {
         const int64_t RM = (int64_t)R * max_tokens;
         d.row = base + (uint64_t)s.grow * (uint64_t)H * (FP8 ? 1 : 2);
-        if (FP8) d.scale = sbase + (uint64_t)((int64_t)k.le * (H / 128) * RM + s.slot) * 4;
         if (slab == 0 && j == 0) {
             ((int32_t*)info)[s.grow] = t;
             sc.row_src[(int64_t)k.e * RM + s.slot] = r * max_tokens + t;
@@ -379,9 +388,17 @@ __device__ __forceinline__ bool pack_token(const uint64_t* __restrict__ tbl, con
     return true;
 }
 
-// fp8, variant 0: a lane owns 16 consecutive elements (32 B in, 16 B out),
-// a 128-element scale group is 8 lanes.
-template <bool NTL, bool NTS>
+// fp8: a lane owns 16 consecutive elements (32 B in, 16 B out), a 128-element
+// scale group is 8 lanes.  The group's scales go to the token's row of
+// scale_stage (contiguous); scale_transpose_kernel moves them into the
+// column-major output with coalesced stores (writing them there from here would
+// be 4-byte stores 16 KB apart).
+//   NATIVE  false: the arithmetic of the reference's PyTorch statement as CPU
+//           PyTorch runs it, `448.0 / amax` = reciprocal times 448 and
+//           `amax / 448.0` a true division (mooncake_ep_buffer.py:699-702);
+//           true: the reference kernel's own, an IEEE quotient 448 / amax and
+//           amax * (1 / 448) (mooncake_ep_kernel.cu:184, :252).
+template <bool NTL, bool NATIVE>
 __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restrict__ tbl,
                                                         RoutingScratch sc, DispatchSource src,
                                                         float* __restrict__ scale_stage, int R, int E, int K,
@@ -428,10 +445,9 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
 #pragma unroll
     for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(f[j]));
     amax = group_max<8>(amax);
-    // the arithmetic of CPU PyTorch for `448.0 / amax` (reciprocal, then times
-    // 448) and `amax / 448.0` (true division), both correctly rounded
-    const float scale = (1.0f / amax) * 448.0f;
-    const float scale_inv = amax / 448.0f;
+    // every division here is the compiler's correctly rounded sequence
+    const float scale = NATIVE ? 448.0f / amax : (1.0f / amax) * 448.0f;
+    const float scale_inv = NATIVE ? amax * (1.0f / 448.0f) : amax / 448.0f;
     uint32_t o[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -440,112 +456,18 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
         o[j] = (uint32_t)w;
     }
     const uint4 out = make_uint4(o[0], o[1], o[2], o[3]);
-    const int64_t scale_off = (int64_t)(elem0 >> 7) * ((int64_t)R * max_tokens) * 4;
-    const bool scale_lane = active && ((lane & 7) == 0);
-    // staged: the token's scales go to one contiguous row, a second kernel
-    // moves them into the column-major output with coalesced stores
-    if (scale_stage != nullptr && scale_lane)
+    if (active && (lane & 7) == 0)
         scale_stage[((int64_t)r * max_tokens + t) * (H >> 7) + (elem0 >> 7)] = scale_inv;
-    const bool scatter_scales = scale_lane && scale_stage == nullptr;
 
     for (int k = 0; k < K; ++k) {
         const uint64_t row = read_lane_u64(dst.row, k * sel_lanes);
-        const uint64_t sc = read_lane_u64(dst.scale, k * sel_lanes);
         if (row == 0) continue;
-        if (active) store16<NTS>((void*)(row + elem0), out);
-        if (scatter_scales) *(float*)(sc + scale_off) = scale_inv;
-    }
-}
-
-// fp8, variant 1: a lane owns two 8-element pieces 512 elements apart, so both
-// 16-byte loads of a wave are unit-stride; a scale group is 16 lanes and the
-// stores are 8 bytes per lane.
-template <bool NTL, bool NTS>
-__global__ __launch_bounds__(512) void pack_fp8_split_kernel(const uint64_t* __restrict__ tbl,
-                                                              RoutingScratch sc, DispatchSource src,
-                                                              float* __restrict__ scale_stage, int R, int E, int K,
-                                                              int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
-                                                              int total_tasks) {
-    const int lane = wave_lane();
-    int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
-    if (task >= total_tasks) return;
-    if (up.carried) {
-        // the first E waves of the launch do the prefix pass (it needs the unit counts only)
-        __shared__ int lds_pre[kMaxPackWaves * (kMaxSummedUnits + 1)];
-        if (task < E) {
-            prefix_expert(tbl, sc, R, E, max_tokens, up.per_rank, up.total, task,
-                          lds_pre + (threadIdx.x >> 6) * (kMaxSummedUnits + 1));
-            return;
-        }
-        task -= E;
-    }
-    const int n = task / slabs, s = task - n * slabs;
-    const int r = n / Tgrid, t = n - r * Tgrid;
-    const char* xbase;
-    const int64_t* idx_row;
-    if (!pack_token(tbl, src, R, K, H, r, t, &xbase, &idx_row)) return;
-
-    int elem[2];
-    bool active[2];
-    uint4 v[2];
-#pragma unroll
-    for (int p = 0; p < 2; ++p) {
-        elem[p] = s * 1024 + p * 512 + lane * 8;
-        active[p] = elem[p] < H;
-        v[p] = make_uint4(0, 0, 0, 0);
-        if (active[p]) v[p] = load16<NTL>(xbase + (int64_t)elem[p] * 2);
-    }
-    const PackDest dst = pack_destination<true>(tbl, sc, idx_row, R, E, K, max_tokens, H, up, r, t, s, lane);
-    const int sel_lanes = sel_stride(up, K);   // selection k's destination sits in lane k * sel_lanes
-
-    uint2 out[2];
-    float scale_inv[2];
-#pragma unroll
-    for (int p = 0; p < 2; ++p) {
-        const uint32_t u[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
-        float f[8];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            f[2 * j] = bf16_lo(u[j]);
-            f[2 * j + 1] = bf16_hi(u[j]);
-        }
-        float amax = 1e-4f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(f[j]));
-        amax = group_max<16>(amax);
-        const float scale = (1.0f / amax) * 448.0f;
-        scale_inv[p] = amax / 448.0f;
-        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0] * scale, f[1] * scale, 0, false);
-        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2] * scale, f[3] * scale, w0, true);
-        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4] * scale, f[5] * scale, 0, false);
-        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6] * scale, f[7] * scale, w1, true);
-        out[p] = make_uint2((uint32_t)w0, (uint32_t)w1);
-    }
-    const int64_t RM4 = (int64_t)R * max_tokens * 4;
-    const bool scale_lane = (lane & 15) == 0;
-    if (scale_stage != nullptr && scale_lane) {
-#pragma unroll
-        for (int p = 0; p < 2; ++p)
-            if (active[p]) scale_stage[((int64_t)r * max_tokens + t) * (H >> 7) + (elem[p] >> 7)] = scale_inv[p];
-    }
-    const bool scatter_scales = scale_lane && scale_stage == nullptr;
-
-    for (int k = 0; k < K; ++k) {
-        const uint64_t row = read_lane_u64(dst.row, k * sel_lanes);
-        const uint64_t sc = read_lane_u64(dst.scale, k * sel_lanes);
-        if (row == 0) continue;
-#pragma unroll
-        for (int p = 0; p < 2; ++p) {
-            if (active[p]) {
-                store8<NTS>((void*)(row + elem[p]), out[p]);
-                if (scatter_scales) *(float*)(sc + (int64_t)(elem[p] >> 7) * RM4) = scale_inv[p];
-            }
-        }
+        if (active) store16<false>((void*)(row + elem0), out);
     }
 }
 
 // bf16: plain row copy, two unit-stride 16-byte pieces per lane.
-template <bool NTL, bool NTS>
+template <bool NTL>
 __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restrict__ tbl,
                                                          RoutingScratch sc, DispatchSource src,
                                                          float* __restrict__ /*scale_stage*/, int R, int E, int K,
@@ -589,7 +511,7 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
         if (row == 0) continue;
 #pragma unroll
         for (int p = 0; p < 2; ++p)
-            if (active[p]) store16<NTS>((void*)(row + off[p]), v[p]);
+            if (active[p]) store16<false>((void*)(row + off[p]), v[p]);
     }
 }
 
@@ -627,21 +549,16 @@ __global__ __launch_bounds__(kTransposeWaves * 64) void scale_transpose_kernel(
     int carry = 0, e = -1, chunk = 0, count = 0;
     auto piece = [&](int e0, int c) {
         const int n = (c + 63) >> 6;
-        int incl = n;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const int up = __shfl_up(incl, d);
-            if (lane >= d) incl += up;
-        }
+        const int incl = wave_scan_inclusive(n);
         const int begin = carry + incl - n;
         const unsigned long long owns = __ballot(n > 0 && begin <= target && target < begin + n);
         if (owns) {
             const int l = __builtin_ctzll(owns);
             e = e0 + l;
-            chunk = target - __shfl(begin, l);
-            count = __shfl(c, l);
+            chunk = target - __builtin_amdgcn_readlane(begin, l);
+            count = __builtin_amdgcn_readlane(c, l);
         }
-        carry += __shfl(incl, 63);
+        carry += __builtin_amdgcn_readlane(incl, 63);
     };
 #pragma unroll
     for (int j = 0; j < kPre; ++j)
@@ -694,6 +611,7 @@ __global__ __launch_bounds__(kTransposeWaves * 64) void scale_transpose_kernel(
 // src_info; each row finds its k in the token's top-k list and leaves the
 // row's address and weight there.  Experts on ranks the owner sees as
 // inactive, and rows of ranks that take no part, leave no route.
+template <bool PACKED>
 __global__ __launch_bounds__(256) void resolve_kernel(const uint64_t* __restrict__ tbl,
                                                        CombineRoute* __restrict__ routes, uint32_t stamp, int R,
                                                        int E, int K, int H, int max_tokens, int total_tasks) {
@@ -734,7 +652,7 @@ __global__ __launch_bounds__(256) void resolve_kernel(const uint64_t* __restrict
             for (int j = 0; j < 4; ++j) {
                 if (cand[j] == (int64_t)e) {
                     CombineRoute rt;
-                    rt.src = row0 + (uint64_t)i * H * 2;
+                    rt.src = PACKED ? (((uint64_t)e << 32) | (uint32_t)(begin + i)) : row0 + (uint64_t)i * H * 2;
                     rt.weight = wt[j];
                     rt.stamp = stamp;
                     rts[(int64_t)t * K + k0 + j] = rt;
@@ -860,6 +778,144 @@ __device__ __forceinline__ uint32_t scale_round_twice(float a, float b, float s,
     return pack_bf16_rne(bf16_lo(once) * f, bf16_hi(once) * f);
 }
 
+// Combine straight from the packed layout dispatch wrote: what cast_back_kernel followed by
+// reduce_kernel computes, without the bf16 expert rows in between.  Every source row is turned, in
+// registers, into exactly what the consumer would have stored -
+//     bf16( bf16( f32(fp8) * scale ) * factor[expert] ),  both roundings to nearest even
+// (per_token_cast_back, mooncake-wheel/tests/ep_test_utils.py:50-53, and the mock expert of
+// mooncake-ep/tests/test_ep_grid.py:168-173; a bf16 payload takes the factor alone) - and then
+// enters the fp32 fused multiply-add chain in k order (mooncake_ep_kernel.cu:711-753), so the result
+// is bit for bit that of the two-kernel path.
+//
+// One wave per (token, slab): 1024 elements of an fp8 payload (16 payload bytes and one scale per lane
+// and row; a 128-element scale group is 8 lanes, and the scales of a row sit R*max floats apart in the
+// column-major layout), 512 elements of a bf16 payload.  Lanes 0..K-1 find the K rows as reduce_kernel
+// does; a masked, inactive or unknown selection reads the zero row with weight 0.
+template <int KMAX, bool FP8, bool FACTOR, bool DIRECT>
+__global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __restrict__ tbl,
+                                                             const CombineRoute* __restrict__ routes, uint32_t stamp,
+                                                             RoutingScratch sc, CombineSource cs,
+                                                             const void* __restrict__ zero_row,
+                                                             const float* __restrict__ factor, int R, int E, int K,
+                                                             int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
+                                                             int total_tasks) {
+    constexpr int kSlab = FP8 ? 1024 : 512;
+    constexpr int kLaneElems = kSlab / 64;
+    const int lane = wave_lane();
+    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    if (task >= total_tasks) return;
+    const int n = task / slabs, s = task - n * slabs;
+    const int r = n / Tgrid, t = n - r * Tgrid;
+    const int T = cs.tokens >= 0 ? cs.tokens : (int)tbl[CF_NUM_TOKENS * R + r];
+    if (t >= T) return;
+    char* orow = (char*)rank_ptr(tbl, cs.out, CF_OUT, R, r) + (int64_t)t * H * 2;
+    const int64_t RM = (int64_t)R * max_tokens;
+    const int G = H >> 7, L = E / R;
+
+    // lanes 0..K-1: where the selection's row, its scales and its factor are
+    uint64_t src = (uint64_t)zero_row, ssrc = (uint64_t)zero_row;
+    float w = 0.0f, f = 1.0f;
+    int sstride = 0;                     // bytes between a row's consecutive scale groups (0: the zero row)
+    {
+        int e = 0, slot = 0;
+        bool ok = false;
+        float wl = 0.0f;
+        if (DIRECT) {
+            const int64_t* idx_row = (const int64_t*)rank_ptr(tbl, cs.topk_idx, CF_TOPK_IDX, R, r) + (int64_t)t * K;
+            const float* w_row = (const float*)rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (int64_t)t * K;
+            wl = w_row[lane < K ? lane : 0];
+            const int32_t* active = (const int32_t*)tbl[CF_ACTIVE * R + r];
+            const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, up, r, t, lane);
+            const int ub = sc.ubegin[(int64_t)k.unit * E + k.e];
+            const int live = active[k.q];                      // skip experts on inactive ranks
+            const SelRow sr = selection_row(k, ub, R, max_tokens);
+            ok = sr.ok && live != 0;
+            e = k.e;
+            slot = sr.slot;
+        } else {
+            uint4 rt = make_uint4(0, 0, 0, 0);
+            if (lane < K) rt = *(const uint4*)(routes + ((int64_t)r * max_tokens + t) * K + lane);
+            ok = (lane < K) && (rt.w == stamp) && (int)rt.y < E && (int64_t)rt.x < RM;
+            e = ok ? (int)rt.y : 0;
+            slot = ok ? (int)rt.x : 0;
+            wl = __uint_as_float(rt.z);
+        }
+        const int q = e / L, le = e - q * L;
+        const uint64_t base = tbl[CF_X * R + q];
+        const uint64_t sbase = FP8 ? tbl[CF_SCALES * R + q] : 0;
+        const float fe = FACTOR ? factor[e] : 1.0f;
+        if (ok && base != 0 && (!FP8 || sbase != 0)) {
+            const int64_t grow = (int64_t)le * RM + slot;
+            src = base + (uint64_t)grow * (uint64_t)H * (FP8 ? 1 : 2);
+            if (FP8) {
+                ssrc = sbase + (uint64_t)((int64_t)le * G * RM + slot) * 4;
+                sstride = (int)(RM * 4);
+            }
+            w = wl;
+            f = fe;
+        }
+    }
+
+    const int elem = s * kSlab + lane * kLaneElems;
+    const bool on = elem < H;
+    const int64_t poff = on ? (int64_t)elem * (FP8 ? 1 : 2) : 0;
+    const int group = on ? (elem >> 7) : 0;
+
+    uint4 v[KMAX];
+    float sv[KMAX], wk[KMAX], fk[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        const uint64_t p = read_lane_u64(src, k);
+        wk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k));
+        fk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), k));
+        v[k] = load16<true>((const void*)(p + poff));
+        if (FP8) {
+            const uint64_t sp = read_lane_u64(ssrc, k);
+            const int st = __builtin_amdgcn_readlane(sstride, k);
+            sv[k] = *(const float*)(sp + (int64_t)group * st);
+        } else {
+            sv[k] = 1.0f;
+        }
+    }
+
+    float acc[kLaneElems];
+#pragma unroll
+    for (int j = 0; j < kLaneElems; ++j) acc[j] = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        const uint32_t u[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (FP8) {
+                typedef float f2 __attribute__((ext_vector_type(2)));
+                const f2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)u[j], false);
+                const f2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)u[j], true);
+                uint32_t lo = pack_bf16_rne(a.x * sv[k], a.y * sv[k]);
+                uint32_t hi = pack_bf16_rne(b.x * sv[k], b.y * sv[k]);
+                if (FACTOR) {
+                    lo = pack_bf16_rne(bf16_lo(lo) * fk[k], bf16_hi(lo) * fk[k]);
+                    hi = pack_bf16_rne(bf16_lo(hi) * fk[k], bf16_hi(hi) * fk[k]);
+                }
+                acc[4 * j + 0] = __builtin_fmaf(bf16_lo(lo), wk[k], acc[4 * j + 0]);
+                acc[4 * j + 1] = __builtin_fmaf(bf16_hi(lo), wk[k], acc[4 * j + 1]);
+                acc[4 * j + 2] = __builtin_fmaf(bf16_lo(hi), wk[k], acc[4 * j + 2]);
+                acc[4 * j + 3] = __builtin_fmaf(bf16_hi(hi), wk[k], acc[4 * j + 3]);
+            } else {
+                uint32_t x = u[j];
+                if (FACTOR) x = pack_bf16_rne(bf16_lo(x) * fk[k], bf16_hi(x) * fk[k]);
+                acc[2 * j + 0] = __builtin_fmaf(bf16_lo(x), wk[k], acc[2 * j + 0]);
+                acc[2 * j + 1] = __builtin_fmaf(bf16_hi(x), wk[k], acc[2 * j + 1]);
+            }
+        }
+    }
+    if (!on) return;
+    uint32_t o[kLaneElems / 2];
+#pragma unroll
+    for (int j = 0; j < kLaneElems / 2; ++j) o[j] = pack_bf16_rne(acc[2 * j], acc[2 * j + 1]);
+    store16<true>(orow + (int64_t)elem * 2, make_uint4(o[0], o[1], o[2], o[3]));
+    if (FP8) store16<true>(orow + (int64_t)elem * 2 + 16, make_uint4(o[4], o[5], o[6], o[7]));
+}
+
 // Work list of the cast-back kernel: which (expert, row chunk) each chunk
 // number is, from the packed_recv_count tensors alone; map[0].x is the number
 // of chunks.  Per block: a thread per expert fetches the count, one wave scans
@@ -894,14 +950,9 @@ __global__ __launch_bounds__(1024) void cast_chunks_kernel(const uint64_t* __res
         for (int e0 = 0; e0 < E; e0 += 64) {
             const int ee = e0 + lane;
             const int n = (ee < E) ? (lds_count[ee] + kCastRows - 1) / kCastRows : 0;
-            int incl = n;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int up = __shfl_up(incl, d);
-                if (lane >= d) incl += up;
-            }
+            const int incl = wave_scan_inclusive(n);
             if (ee < E) lds_begin[ee] = carry + incl - n;
-            carry += __shfl(incl, 63);
+            carry += __builtin_amdgcn_readlane(incl, 63);
         }
         if (lane == 0) {
             lds_begin[E] = carry;
@@ -1146,22 +1197,23 @@ hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const Di
                        const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
                        hipStream_t stream) {
     // measured: streaming loads pay when a token's row goes to many experts, not when it goes to a few
-    const int pack_nt = t.pack_nt >= 0 ? t.pack_nt : (d.K > 4 ? 1 : 0);
-    const bool ntl = pack_nt & 1, nts = pack_nt & 2;
-    float* stage = (use_fp8 && t.scale_mode == 1) ? scale_stage : nullptr;
+    // (and streaming stores never did)
+    const bool ntl = t.pack_nt >= 0 ? (t.pack_nt & 1) != 0 : d.K > 4;
+    if (use_fp8 && scale_stage == nullptr) return hipErrorInvalidValue;
     hipError_t err = hipSuccess;
     if (run_pack) {
-#define MCEP_PACK(KERN)                                                                          \
-    (ntl ? (nts ? launch_pack_t(KERN<true, true>, d_tbl, sc, src, stage, d, t, stream)           \
-                : launch_pack_t(KERN<true, false>, d_tbl, sc, src, stage, d, t, stream))         \
-         : (nts ? launch_pack_t(KERN<false, true>, d_tbl, sc, src, stage, d, t, stream)          \
-                : launch_pack_t(KERN<false, false>, d_tbl, sc, src, stage, d, t, stream)))
-        if (!use_fp8) err = MCEP_PACK(pack_bf16_kernel);
-        else if (t.pack_variant == 1) err = MCEP_PACK(pack_fp8_split_kernel);
-        else err = MCEP_PACK(pack_fp8_kernel);
-#undef MCEP_PACK
+        if (!use_fp8)
+            err = ntl ? launch_pack_t(pack_bf16_kernel<true>, d_tbl, sc, src, scale_stage, d, t, stream)
+                      : launch_pack_t(pack_bf16_kernel<false>, d_tbl, sc, src, scale_stage, d, t, stream);
+        else if (t.fp8_arith == 1)
+            err = ntl ? launch_pack_t(pack_fp8_kernel<true, true>, d_tbl, sc, src, scale_stage, d, t, stream)
+                      : launch_pack_t(pack_fp8_kernel<false, true>, d_tbl, sc, src, scale_stage, d, t, stream);
+        else
+            err = ntl ? launch_pack_t(pack_fp8_kernel<true, false>, d_tbl, sc, src, scale_stage, d, t, stream)
+                      : launch_pack_t(pack_fp8_kernel<false, false>, d_tbl, sc, src, scale_stage, d, t, stream);
     }
-    if (err != hipSuccess || stage == nullptr || !run_finish) return err;
+    if (err != hipSuccess || !use_fp8 || !run_finish) return err;
+    float* stage = scale_stage;
     const int G = d.H / 128;
     const int parts = (G + kTransposeGroups - 1) / kTransposeGroups;
     // every selection is at most one row, and each expert has at most one partly filled chunk
@@ -1174,15 +1226,19 @@ hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const Di
     return hipGetLastError();
 }
 
-hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, const Dims& d,
+hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, bool packed, const Dims& d,
                           const Tuning& /*t*/, hipStream_t stream) {
     const long long total = (long long)d.E * d.R;
     if (total <= 0) return hipSuccess;
     if (total > 0x7fffffffll) return hipErrorInvalidValue;
     const int wpb = 4;
     const int blocks = (int)((total + wpb - 1) / wpb);
-    hipLaunchKernelGGL(resolve_kernel, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_routes, stamp, d.R, d.E, d.K,
-                       d.H, d.max_tokens, (int)total);
+    if (packed)
+        hipLaunchKernelGGL(resolve_kernel<true>, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_routes, stamp, d.R,
+                           d.E, d.K, d.H, d.max_tokens, (int)total);
+    else
+        hipLaunchKernelGGL(resolve_kernel<false>, dim3(blocks), dim3(wpb * 64), 0, stream, d_tbl, d_routes, stamp, d.R,
+                           d.E, d.K, d.H, d.max_tokens, (int)total);
     return hipGetLastError();
 }
 
@@ -1239,6 +1295,43 @@ hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, ui
     if (d.K <= 12) MCEP_K(12);
     MCEP_K(16);
 #undef MCEP_K
+}
+
+template <int KMAX, bool FP8, bool FACTOR, bool DIRECT>
+static hipError_t launch_reduce_packed_t(const ReduceLaunch& rl, const float* d_factor, const Dims& d, const Tuning& t,
+                                         hipStream_t stream) {
+    const int slab = FP8 ? 1024 : 512;
+    const int slabs = (d.H + slab - 1) / slab;
+    const long long total = (long long)d.R * d.Tgrid * slabs;
+    if (total <= 0) return hipSuccess;
+    if (total > 0x7fffffffll) return hipErrorInvalidValue;
+    const int wpb = clamp_waves(t.combine_waves);
+    const int blocks = (int)((total + wpb - 1) / wpb);
+    hipLaunchKernelGGL((reduce_packed_kernel<KMAX, FP8, FACTOR, DIRECT>), dim3(blocks), dim3(wpb * 64), 0, stream,
+                       rl.d_tbl, rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d_factor, d.R, d.E, d.K,
+                       d.max_tokens, d.H, d.plan, slabs, d.Tgrid, (int)total);
+    return hipGetLastError();
+}
+
+hipError_t launch_reduce_packed(const uint64_t* d_tbl, const CombineRoute* d_routes, uint32_t stamp,
+                                const RoutingScratch& sc, bool direct, const CombineSource& src, const void* d_zero_row,
+                                const float* d_factor, bool use_fp8, const Dims& d, const Tuning& t, hipStream_t stream) {
+    const ReduceLaunch rl{d_tbl, d_routes, stamp, sc, src, d_zero_row};
+    const bool fac = d_factor != nullptr;
+#define MCEP_P4(KMAX, FP8, FACTOR)                                                                   \
+    (direct ? launch_reduce_packed_t<KMAX, FP8, FACTOR, true>(rl, d_factor, d, t, stream)            \
+            : launch_reduce_packed_t<KMAX, FP8, FACTOR, false>(rl, d_factor, d, t, stream))
+#define MCEP_PK(KMAX)                                                                                \
+    do {                                                                                             \
+        if (use_fp8) return fac ? MCEP_P4(KMAX, true, true) : MCEP_P4(KMAX, true, false);            \
+        return fac ? MCEP_P4(KMAX, false, true) : MCEP_P4(KMAX, false, false);                       \
+    } while (0)
+    if (d.K <= 2) MCEP_PK(2);
+    if (d.K <= 4) MCEP_PK(4);
+    if (d.K <= 8) MCEP_PK(8);
+    MCEP_PK(16);
+#undef MCEP_PK
+#undef MCEP_P4
 }
 
 long long cast_back_chunks(long long max_rows, int num_experts) {

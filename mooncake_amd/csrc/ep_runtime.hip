@@ -518,10 +518,18 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     return MC_EP_OK;
 }
 
+// What combine reads its rows from: bf16 expert outputs (the reference's combine), or, for the packed
+// combine, the payload dispatch wrote (fp8 with scales, or bf16) times an optional per-expert factor.
+struct PackedSource {
+    bool packed = false;
+    const uint64_t* scales = nullptr;   // per-rank addresses; null: the payload is bf16
+    const float* factor = nullptr;      // device f32 [num_experts]; null: no factor
+};
+
 int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_idx, const uint64_t* topk_weights,
                        const uint64_t* src_info, const uint64_t* layout_range, const uint64_t* active_ranks,
                        const int32_t* num_tokens, int hidden, int num_topk, int max_tokens, int num_experts,
-                       const uint64_t* out, int phases, hipStream_t stream) {
+                       const uint64_t* out, int phases, hipStream_t stream, const PackedSource& ps = PackedSource()) {
     const int R = w->R;
     if (int rc = check_dims(w, hidden, num_topk, max_tokens, num_experts)) return rc;
     MC_ASSERT(x != nullptr && topk_idx != nullptr && topk_weights != nullptr && num_tokens != nullptr);
@@ -536,6 +544,8 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
             MC_ASSERT(out[r] != 0);
         }
         if (x[r] != 0) MC_ASSERT(src_info[r] != 0 && layout_range[r] != 0);
+        if (x[r] != 0 && ps.scales != nullptr) MC_ASSERT(ps.scales[r] != 0);
+        tbl[CF_SCALES * R + r] = (ps.scales != nullptr && x[r] != 0) ? ps.scales[r] : 0;
         tbl[CF_X * R + r] = x[r];
         tbl[CF_TOPK_IDX * R + r] = topk_idx[r];
         tbl[CF_TOPK_W * R + r] = topk_weights[r];
@@ -591,10 +601,13 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
             if (cap.active)
                 MC_HIP(launch_fill_u32(w->d_routes, 0u, (size_t)R * max_tokens * num_topk * (sizeof(CombineRoute) / 4),
                                        stream));
-            MC_HIP(launch_resolve(d_tbl, w->d_routes, w->stamp, d, w->tuning, stream));
+            MC_HIP(launch_resolve(d_tbl, w->d_routes, w->stamp, ps.packed, d, w->tuning, stream));
         }
     }
-    if (phases & MC_EP_PHASE_DATA)
+    if ((phases & MC_EP_PHASE_DATA) && ps.packed)
+        MC_HIP(launch_reduce_packed(d_tbl, w->d_routes, w->stamp, routing_scratch(w), direct, src, w->d_zero_row,
+                                    ps.factor, ps.scales != nullptr, d, w->tuning, stream));
+    else if (phases & MC_EP_PHASE_DATA)
         MC_HIP(launch_reduce(d_tbl, w->d_routes, w->stamp, routing_scratch(w), direct, src, w->d_zero_row, d,
                              w->tuning, stream));
     return MC_EP_OK;
@@ -907,11 +920,10 @@ int mc_ep_world_set_rank_silent(mc_ep_world_t* w, int rank, int silent) {
 }
 
 static int* option_slot(Tuning& t, const char* name) {
-    if (!strcmp(name, "pack_variant")) return &t.pack_variant;
     if (!strcmp(name, "pack_waves")) return &t.pack_waves;
     if (!strcmp(name, "pack_nt")) return &t.pack_nt;
     if (!strcmp(name, "uniform")) return &t.uniform;
-    if (!strcmp(name, "scale_mode")) return &t.scale_mode;
+    if (!strcmp(name, "fp8_arith")) return &t.fp8_arith;
     if (!strcmp(name, "combine_direct")) return &t.combine_direct;
     if (!strcmp(name, "combine_chunks")) return &t.combine_chunks;
     if (!strcmp(name, "routing_sum")) return &t.routing_sum;
@@ -969,6 +981,22 @@ int mc_ep_world_combine(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_t
     return world_combine_impl(w, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
                               active_ranks_ptrs, num_combined_tokens, hidden, num_topk, max_tokens, num_experts,
                               combined_x_ptrs, phases, (hipStream_t)stream_ptr);
+}
+
+int mc_ep_world_combine_packed(mc_ep_world_t* w, const uint64_t* recv_x_ptrs, const uint64_t* recv_scales_ptrs,
+                               uint64_t expert_factor_ptr, const uint64_t* topk_idx_ptrs,
+                               const uint64_t* topk_weights_ptrs, const uint64_t* src_info_ptrs,
+                               const uint64_t* layout_range_ptrs, const uint64_t* active_ranks_ptrs,
+                               const int32_t* num_combined_tokens, int hidden, int num_topk, int max_tokens,
+                               int num_experts, const uint64_t* combined_x_ptrs, int phases, uint64_t stream_ptr) {
+    MC_ASSERT(w != nullptr);
+    PackedSource ps;
+    ps.packed = true;
+    ps.scales = recv_scales_ptrs;
+    ps.factor = (const float*)expert_factor_ptr;
+    return world_combine_impl(w, recv_x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
+                              active_ranks_ptrs, num_combined_tokens, hidden, num_topk, max_tokens, num_experts,
+                              combined_x_ptrs, phases, (hipStream_t)stream_ptr, ps);
 }
 
 int mc_ep_world_cast_back(mc_ep_world_t* w, const uint64_t* recv_x_ptrs, const uint64_t* recv_scales_ptrs,

@@ -102,6 +102,25 @@ class World:
                 _lib.check(rc)
         return call
 
+    def prepare_combine_packed(self, recv_x_ptrs, recv_scales_ptrs, expert_factor_ptr, topk_idx_ptrs,
+                               topk_weights_ptrs, src_info_ptrs, layout_range_ptrs, active_ranks_ptrs,
+                               num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank, num_experts,
+                               combined_x_ptrs):
+        """Combine straight from dispatch's packed output (fp8 payload with scales, or bf16 when
+        recv_scales_ptrs is None) times expert_factor[expert] (0: none): cast_back + combine in one."""
+        u = _lib.u64_array
+        fn = _lib.lib().mc_ep_world_combine_packed
+        args = (self._h, u(recv_x_ptrs), u(recv_scales_ptrs) if recv_scales_ptrs is not None else None,
+                int(expert_factor_ptr), u(topk_idx_ptrs), u(topk_weights_ptrs), u(src_info_ptrs),
+                u(layout_range_ptrs), u(active_ranks_ptrs), _lib.i32_array(num_combined_tokens), hidden, num_topk,
+                num_max_dispatch_tokens_per_rank, num_experts, u(combined_x_ptrs))
+
+        def call(stream_ptr: int, phases: int = _lib.PHASE_ALL) -> None:
+            rc = fn(*args, phases, stream_ptr)
+            if rc:
+                _lib.check(rc)
+        return call
+
     def dispatch(self, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
                  num_experts, use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
                  layout_range_ptrs, stream_ptr: int, phases: int = _lib.PHASE_ALL) -> None:

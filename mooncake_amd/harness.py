@@ -121,6 +121,28 @@ class WorldHarness:
             self._prepared[key] = call
         call(self._stream(stream), phases)
 
+    def combine_packed(self, factor_per_expert: Optional[torch.Tensor] = None, phases: int = _lib.PHASE_ALL,
+                       stream: Optional[torch.cuda.Stream] = None, present: Optional[Sequence[int]] = None) -> None:
+        """combined = combine(cast_back(recv_x, factor)) in one kernel, reading dispatch's packed output."""
+        c = self.cfg
+        R = c.num_ranks
+        self._factor = None if factor_per_expert is None else \
+            factor_per_expert.to(device=self.device, dtype=torch.float32).contiguous()
+        fptr = 0 if self._factor is None else self._factor.data_ptr()
+        key = ("combine_packed", None if present is None else tuple(present), self.recv_x.data_ptr(),
+               self.combined.data_ptr(), self.src_info.data_ptr(), fptr)
+        call = self._prepared.get(key)
+        if call is None:
+            nt = [n if (present is None or present[r]) else 0 for r, n in enumerate(self.num_tokens)]
+            call = self.world.prepare_combine_packed(
+                self._ptrs(self.recv_x, R, present),
+                self._ptrs(self.recv_scales_phys, R, present) if c.use_fp8 else None, fptr,
+                self._ptrs(self.topk_idx, R), self._ptrs(self.topk_weights, R), self._ptrs(self.src_info, R),
+                self._ptrs(self.layout_range, R), self._ptrs(self.active_ranks, R), nt, c.hidden, c.num_topk,
+                c.max_tokens, c.num_experts, self._ptrs(self.combined, R))
+            self._prepared[key] = call
+        call(self._stream(stream), phases)
+
     # ------------------------------------------------------------------
     def recv_x_typed(self) -> torch.Tensor:
         return self.recv_x.view(torch.float8_e4m3fn) if self.cfg.use_fp8 else self.recv_x.view(torch.bfloat16)

@@ -151,12 +151,23 @@ ORACLE_API void oracle_f32_to_bf16(const float* in, uint16_t* out, int64_t n) {
  * `tensor / 448.0` is a true IEEE division (K:252 multiplies by 1/448
  * instead).  tests/test_oracle_fp8.py pins both against torch itself.
  * NaN elements do not raise amax (fmaxf, K:247); they encode as fp8 NaN. */
+/* Which of the reference's two statements of the scale arithmetic is restated: 0 (default) the PyTorch
+ * one above, 1 the CUDA kernel's own - scale = 448 / amax as one IEEE division (K:252; nvcc divides
+ * correctly rounded unless told otherwise, and the reference's build does not tell it) and the stored
+ * scale amax * (1 / 448) with the constant folded at compile time (K:184, K:252).  The two differ in
+ * the last bit of either scale for about a quarter of all amax values.
+ * tests/test_oracle_fp8.py pins mode 1 against numpy's float32 division and product. */
+static int g_fp8_arith = 0;
+
+ORACLE_API void oracle_set_fp8_arith(int mode) { g_fp8_arith = mode ? 1 : 0; }
+
 static void quantise_row(const uint16_t* x, int H, uint8_t* q, float* scales, int64_t scale_stride) {
+    const int native = g_fp8_arith;
     for (int g = 0; g < H / 128; ++g) {
         float amax = 1e-4f;
         for (int j = 0; j < 128; ++j) amax = fmaxf(amax, fabsf(bf16_to_f32(x[g * 128 + j])));
-        float scale = (1.0f / amax) * 448.0f;
-        float scale_inv = amax / 448.0f;
+        const float scale = native ? 448.0f / amax : (1.0f / amax) * 448.0f;
+        const float scale_inv = native ? amax * (1.0f / 448.0f) : amax / 448.0f;
         for (int j = 0; j < 128; ++j) q[g * 128 + j] = f32_to_e4m3fn(bf16_to_f32(x[g * 128 + j]) * scale);
         scales[(int64_t)g * scale_stride] = scale_inv;
     }

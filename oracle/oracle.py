@@ -69,6 +69,11 @@ def f32_to_bf16_bits(v: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def set_fp8_arith(mode: int) -> None:
+    """0: the scale arithmetic of the reference's PyTorch statement (default); 1: the CUDA kernel's own."""
+    lib().oracle_set_fp8_arith(int(mode))
+
+
 def quantise_rows(x: torch.Tensor):
     """x [rows, H] bf16 -> (payload uint8 [rows, H], scales f32 [rows, H/128])."""
     assert x.dtype == torch.bfloat16 and x.dim() == 2 and x.size(1) % 128 == 0

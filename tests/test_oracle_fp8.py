@@ -130,6 +130,60 @@ def test_row_quantiser_all_bf16_values(oracle):
         assert torch.equal(s.view(torch.int32), s_ref.view(torch.int32))
 
 
+def kernel_formula(x: torch.Tensor):
+    """The reference kernel's own arithmetic (mooncake_ep_kernel.cu:184, :247-260): one IEEE division
+    448 / amax for the payload scale, amax * (1/448) with the float constant for the stored scale,
+    executed by numpy in float32; the cast itself by torch."""
+    import numpy as np
+    m, n = x.shape
+    xv = x.float().view(m, -1, 128)
+    amax = xv.abs().amax(dim=2).clamp(1e-4).numpy().astype(np.float32)
+    scale = (np.float32(448.0) / amax).astype(np.float32)
+    scale_inv = (amax * (np.float32(1.0) / np.float32(448.0))).astype(np.float32)
+    q = (xv * torch.from_numpy(scale).unsqueeze(2)).to(torch.float8_e4m3fn).view(m, n)
+    return q, torch.from_numpy(scale_inv)
+
+
+def test_row_quantiser_in_the_kernels_own_arithmetic(oracle):
+    vals = all_bf16_as_f32()
+    vals = vals[torch.isfinite(vals)]
+    g = torch.Generator().manual_seed(12)
+    pad = (-vals.numel()) % 1024
+    shuffled = torch.cat([vals[torch.randperm(vals.numel(), generator=g)], torch.zeros(pad)]).view(-1, 1024)
+    ordered = torch.cat([vals.sort().values, torch.zeros(pad)]).view(-1, 1024)
+    x = torch.cat([shuffled, ordered, torch.randn(64, 1024, generator=g), torch.randn(16, 1024, generator=g) * 100.0])
+    x = x.to(torch.bfloat16)
+    q_py, s_py = oracle.quantise_rows(x)
+    oracle.set_fp8_arith(1)
+    try:
+        q, s = oracle.quantise_rows(x)
+    finally:
+        oracle.set_fp8_arith(0)
+    q_ref, s_ref = kernel_formula(x)
+    assert torch.equal(q, q_ref.view(torch.uint8))
+    assert torch.equal(s.view(torch.int32), s_ref.view(torch.int32))
+    # the two statements of the reference really are different functions: the stored scale differs in its
+    # last bit for a good part of the groups, and some payload bytes follow the payload scale
+    differ = (s.view(torch.int32) != s_py.view(torch.int32)).float().mean().item()
+    assert 0.05 < differ < 0.6
+    assert (s.view(torch.int32) - s_py.view(torch.int32)).abs().max().item() == 1
+    assert 0 < (q != q_py).float().mean().item() < 0.01
+    # A known answer, worked in exact rational arithmetic: amax = 3.  float32(1/448) = 0x3B124925, and
+    # 3 * that rounds to 0x3BDB6DB8 - the kernel's stored scale - while 3/448 itself rounds to 0x3BDB6DB7,
+    # the PyTorch statement's.  Both give 448/3 -> 0x43155555 or a neighbour, and 3 * scale -> code 0x7E (448).
+    one = torch.zeros(1, 128, dtype=torch.bfloat16)
+    one[0, 0] = 3.0
+    q0, s0 = oracle.quantise_rows(one)
+    oracle.set_fp8_arith(1)
+    try:
+        q1, s1 = oracle.quantise_rows(one)
+    finally:
+        oracle.set_fp8_arith(0)
+    assert s1.view(torch.int32)[0, 0].item() == 0x3BDB6DB8
+    assert s0.view(torch.int32)[0, 0].item() == 0x3BDB6DB7
+    assert q1[0, 0].item() == 0x7E and q0[0, 0].item() == 0x7E
+
+
 def test_nan_elements_do_not_poison_their_group(oracle):
     # the kernel's fmaxf drops NaN from amax (mooncake_ep_kernel.cu:247); the NaN element itself stays NaN
     x = torch.ones(1, 128, dtype=torch.bfloat16) * 2.0
