@@ -22,14 +22,25 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published peak
 METRIC = "dispatch+combine µs & HBM GB/s (% peak), DSV3 decode 128 tok top-8 fp8"
 
-# HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs of
-# this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what
-# the same counter reads for the library's plain copy kernel over 1 GiB
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Workloads not profiled report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("dsv3_decode", "reduce"): int((231475.1 * 2.0 + 57344.0 * 1.0) * 1024),
-    ("dsv3_decode", "pack"): int((30769.1 * 2.0 + 232430.4 * 1.0) * 1024),
-}
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of a kernel as the profiler's counters saw them: the `traffic_bytes` lines of
+    profiles/<workload>_hbm_traffic.txt, which `python -m mooncake_amd.benchmarks.hbm_traffic` writes from two
+    `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter
+    reads for the library's plain copy kernel of known size.  The file records the commit of the library it was
+    measured on, which is passed on; a workload or kernel that was not profiled gives (None, None)."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None, None
+    commit, found = None, None
+    for line in open(path):
+        parts = line.split()
+        if len(parts) >= 2 and parts[0] == "measured_at_commit":
+            commit = parts[1]
+        if len(parts) >= 3 and parts[0] == "traffic_bytes" and parts[1] == kernel:
+            found = int(parts[2])
+    return found, commit
 
 
 def parse_args():
@@ -40,6 +51,8 @@ def parse_args():
     ap.add_argument("--config", default="dsv3_decode")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-flushed", action="store_true", help="skip the cache-flushed timing")
+    ap.add_argument("--no-buffer-api", action="store_true", help="skip the per-rank Buffer API timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget for the cpu_baseline sample")
     ap.add_argument("--kernel-iters", type=int, default=30, help="timed launches per kernel for the roofline figures")
     ap.add_argument("--opt", action="append", default=[], help="library tuning option, name=value")
@@ -125,11 +138,133 @@ def time_back_to_back(call, iters):
     return a.elapsed_time(b) * 1e3 / iters
 
 
+def time_flushed(h, iters, alg):
+    """The reference's timing protocol taken to its strict form: the caches are flushed with 512 MiB before
+    every timed step (its benchmarks flush 256 MB once, after the warm-up: ep_test_utils.py:79-104), 20 warm-ups
+    and `iters` timed steps with an event pair around each call, the first one dropped.  Two kinds of flush,
+    because they leave different cache states behind: a written one (the reference's `cache.zero_()`; its dirty
+    lines are evicted while the timed kernel runs, which the kernel pays for) and a read-only one (clean lines)."""
+    import torch
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device=h.device)
+    flush.zero_()
+    sink = torch.zeros(1, dtype=torch.int64, device=h.device)
+    kinds = {"written": lambda: flush.zero_(),
+             "read_only": lambda: sink.add_(flush.view(torch.int64).sum())}
+    out = {"flush_mib": 512}
+    for name, do_flush in kinds.items():
+        for _ in range(20):
+            h.dispatch()
+            h.combine()
+        marks = []
+        for _ in range(iters + 1):
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+            do_flush()
+            ev[0].record()
+            h.dispatch()
+            ev[1].record()
+            do_flush()
+            ev[2].record()
+            h.combine()
+            ev[3].record()
+            marks.append(ev)
+        torch.cuda.synchronize()
+        d = [m[0].elapsed_time(m[1]) * 1e3 for m in marks[1:]]
+        c = [m[2].elapsed_time(m[3]) * 1e3 for m in marks[1:]]
+        d_us, c_us = sum(d) / len(d), sum(c) / len(c)
+        out[name] = {"dispatch_us": round(d_us, 2), "combine_us": round(c_us, 2),
+                     "pct_of_hbm_peak": round((alg["dispatch"] + alg["combine"]) / (d_us + c_us) / 1e3
+                                              / HBM_PEAK_GBPS * 100, 2),
+                     "dispatch_pct": round(alg["dispatch"] / d_us / 1e3 / HBM_PEAK_GBPS * 100, 2),
+                     "combine_pct": round(alg["combine"] / c_us / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+    return out
+
+
+def time_buffer_api(h, steps, warmup):
+    """The same step driven the way the reference's callers drive it: one `Buffer.dispatch` and one
+    `Buffer.combine` per logical rank (2 x num_ranks calls a step) through the module that replaces
+    `mooncake._ep` (ep_py.cpp:26-46), raw addresses in, (event, hook) out.  Wall clock per step like `value`;
+    `host_us` is the time the calling thread spends inside the calls of a step (hidden behind the GPU when it is
+    below the step time)."""
+    import torch
+    from mooncake_amd import ep
+    cfg = h.cfg
+    R, T, H, K, E, L = cfg.num_ranks, cfg.tokens_per_rank, cfg.hidden, cfg.num_topk, cfg.num_experts, \
+        cfg.num_local_experts
+    nbytes = ep.get_ep_buffer_size_hint(cfg.max_tokens, H, R, E)
+    bufs = [ep.Buffer(r, R, nbytes, False, world=h.world) for r in range(R)]
+    stream = int(torch.cuda.current_stream().cuda_stream)
+    scales = h.recv_scales_phys
+    out = {"binding": ep.BINDING, "calls_per_step": 2 * R}
+    for mode, (async_, hook) in {"async_finish": (True, False), "default": (False, False),
+                                 "return_recv_hook": (False, True)}.items():
+        d = [(h.x[r].data_ptr(), h.topk_idx[r].data_ptr(), h.active_ranks[r].data_ptr(), T, H, K, cfg.max_tokens, E,
+              -1, cfg.use_fp8, h.recv_x[r].data_ptr(), scales[r].data_ptr() if cfg.use_fp8 else 0,
+              h.recv_count[r].data_ptr(), h.src_info[r].data_ptr(), h.layout_range[r].data_ptr(), async_, hook,
+              stream) for r in range(R)]
+        c = [(h.expert_out[r].data_ptr(), h.topk_idx[r].data_ptr(), h.topk_weights[r].data_ptr(),
+              h.src_info[r].data_ptr(), h.layout_range[r].data_ptr(), h.active_ranks[r].data_ptr(), L, T, H, K,
+              cfg.max_tokens, E, -1, False, h.combined[r].data_ptr(), async_, hook, stream) for r in range(R)]
+
+        def step():
+            for name, args in (("dispatch", d), ("combine", c)):
+                res = [getattr(bufs[r], name)(*args[r]) for r in range(R)]
+                for ev, fn in res:          # every rank waits for its own result, as a caller of the reference does
+                    if ev is not None:
+                        ev.current_stream_wait(stream)
+                    if fn is not None:
+                        fn()
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        out[mode] = {"us_per_step": round((t2 - t0) / steps * 1e6, 2), "host_us": round((t1 - t0) / steps * 1e6, 2)}
+    return out
+
+
+def time_python_buffer(h, steps, warmup):
+    """One level up: the Python `Buffer` with the reference wrapper's signature (mooncake_ep_buffer.py:360-535,
+    :538-678), which checks its arguments and allocates the five output tensors of every rank's dispatch with
+    torch.empty inside the call.  In the reference each rank pays that in its own process; here one thread pays
+    it for all ranks, so this figure is host-bound and reported for completeness only."""
+    import torch
+    from mooncake_amd.mooncake_ep_buffer import Buffer, LogicalGroup
+    cfg = h.cfg
+    R = cfg.num_ranks
+    nbytes = Buffer.get_ep_buffer_size_hint(cfg.max_tokens, cfg.hidden, R, cfg.num_experts)
+    bufs = [Buffer(LogicalGroup(h.world, r), nbytes) for r in range(R)]
+    expert_out = [h.expert_out[r] for r in range(R)]
+
+    def step():
+        res = [bufs[r].dispatch(h.x[r], h.topk_idx[r], h.active_ranks[r], cfg.max_tokens, cfg.num_experts, -1,
+                                use_fp8=cfg.use_fp8, async_finish=True) for r in range(R)]
+        for r in range(R):
+            res[r][3].current_stream_wait()
+        outs = [bufs[r].combine(expert_out[r], h.topk_idx[r], h.topk_weights[r], h.active_ranks[r], -1, res[r][2],
+                                async_finish=True, out=h.combined[r]) for r in range(R)]
+        for r in range(R):
+            outs[r][1].current_stream_wait()
+    for _ in range(max(2, warmup // 4)):
+        step()
+    torch.cuda.synchronize()
+    n = max(5, steps // 4)
+    t0 = time.perf_counter()
+    for _ in range(n):
+        step()
+    torch.cuda.synchronize()
+    return {"us_per_step": round((time.perf_counter() - t0) / n * 1e6, 2), "steps": n}
+
+
 def cpu_baseline(cfg, data, bytes_total, budget_s):
     """The oracle (a scalar C restatement, OpenMP over tokens) timed on this
     host's cores on the same workload: whole steps until the budget is spent."""
     import torch
     from oracle import oracle
+    # a one-GPU box's share of its host is 16 cores, whatever os.cpu_count() says there
     threads = min(16, os.cpu_count() or 1)
     oracle.set_threads(threads)
     R = cfg.num_ranks
@@ -249,9 +384,19 @@ def main():
     torch.cuda.synchronize()
     cast_us = ev[0].elapsed_time(ev[-1]) / args.kernel_iters * 1e3
     consumer = {"cast_back_us": round(cast_us, 2), "bytes": cast_bytes, "GBps": round(cast_bytes / cast_us / 1e3, 1)}
+    # the combine fused with that consumer (reads dispatch's payload, same result bit for bit): against the two
+    # kernels it replaces, both timed back to back
+    packed_us = time_back_to_back(h.combine_packed, args.kernel_iters)
+    packed_bytes = S * ((H + H // 128 * 4) if cfg.use_fp8 else 2 * H) + alg["combine"] - S * 2 * H
+    fused = {"cast_back_plus_reduce_us": round(cast_us + red_b2b, 2), "combine_packed_us": round(packed_us, 2),
+             "bytes": packed_bytes, "GBps": round(packed_bytes / packed_us / 1e3, 1),
+             "pct_of_hbm_peak": round(packed_bytes / packed_us / 1e3 / HBM_PEAK_GBPS * 100, 2)}
+    h.dispatch()
+    h.cast_back()
     # the dominant kernel is the one the step spends most time in
     dom = "reduce" if red_us >= pack_us else "pack"
     achieved = kernels[dom]["GBps"]
+    traffic, traffic_at = measured_traffic(cfg.name, dom)
     out = {
         "metric": METRIC,
         "value": round(step_gbps, 1),
@@ -278,10 +423,16 @@ def main():
         "algorithmic_bytes": alg,
         "kernels": kernels,
         "consumer": consumer,
+        "fused_combine": fused,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((cfg.name, dom)) if not opts else None},
+                     "traffic": None if opts else traffic, "traffic_measured_at_commit": None if opts else traffic_at},
     }
+    if not args.no_flushed:
+        out["flushed"] = time_flushed(h, args.kernel_iters, alg)
+    if not args.no_buffer_api:
+        out["buffer_api"] = time_buffer_api(h, args.steps, args.warmup)
+        out["buffer_api"]["python_buffer_async_finish"] = time_python_buffer(h, args.steps, args.warmup)
     if args.copy_calibration > 0:
         nbytes = args.copy_calibration << 20
         src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").fill_(1)

@@ -137,6 +137,7 @@ struct Tuning {
     int combine_waves = 4;     // waves per block in the combine kernel
     int combine_nt = 3;        // bit 0: streaming loads, bit 1: streaming stores
     int routing_sum = 1;       // allow the summed routing plan (see UnitPlan) where the shape permits
+    int comm_stream = 0;       // 1: per-rank rounds always run on the world's communication stream
 };
 
 // Chooses the unit plan for a shape (summed when allowed, the shape permits and there are tokens).

@@ -55,11 +55,33 @@ int fail(int code, const std::string& msg) {
                                            std::to_string(__LINE__) + " '" + hipGetErrorString(e_) + "'");    \
     } while (0)
 
+// Events are reused: a collective needs one or two per round, and creating and destroying them costs
+// more host time than the rest of a per-rank call.  Shared by a world and its rounds, which may outlive it
+// (an EventHandle still held by the caller).
+struct EventPool {
+    std::vector<hipEvent_t> idle;
+    int take(hipEvent_t* out) {
+        if (!idle.empty()) {
+            *out = idle.back();
+            idle.pop_back();
+            return MC_EP_OK;
+        }
+        MC_HIP(hipEventCreateWithFlags(out, hipEventDisableTiming));
+        return MC_EP_OK;
+    }
+    void give(hipEvent_t e) { idle.push_back(e); }
+    ~EventPool() {
+        for (hipEvent_t e : idle) (void)hipEventDestroy(e);
+    }
+};
+
 // One collective call (a "round"): the j-th dispatch (or combine) of every live rank.
 struct Round {
     bool launched = false;
     std::string failure;          // why the round's launch failed, if it did
     hipEvent_t done = nullptr;
+    std::shared_ptr<EventPool> pool;       // where `done` came from and goes back to
+    std::vector<hipStream_t> waited;       // streams that already wait for `done`: a second wait adds nothing
     // A round whose callers all asked for a receive hook is launched in two parts, like the
     // reference's SEND / RECV phases (mooncake_ep_buffer.cpp:303-305, :330-335): the call that
     // completes it enqueues the layout and data kernels, the first hook that is called enqueues the
@@ -67,7 +89,19 @@ struct Round {
     std::function<int()> finish;
     hipStream_t launch_stream = nullptr;
     ~Round() {
-        if (done) (void)hipEventDestroy(done);
+        if (done && pool) pool->give(done);
+        else if (done) (void)hipEventDestroy(done);
+    }
+    // makes `stream` wait for the round's completion, once
+    int make_wait(hipStream_t stream) {
+        for (hipStream_t s : waited)
+            if (s == stream) return MC_EP_OK;
+        if (done == nullptr)
+            return fail(MC_EP_ERR_ASSERT, "Failed: a stream that took no part in the collective asks to wait for "
+                                          "it, and no caller of the round asked for a completion event");
+        MC_HIP(hipStreamWaitEvent(stream, done, 0));
+        waited.push_back(stream);
+        return MC_EP_OK;
     }
 };
 
@@ -105,6 +139,8 @@ struct mc_ep_world {
     // waits for what that stream holds (order_begin).
     hipEvent_t ordered = nullptr;
     hipStream_t ordered_stream = nullptr;                // where the world's last eager sequence ran
+    hipEvent_t fence = nullptr;                          // callers' streams -> launch stream, re-recorded per use
+    std::shared_ptr<EventPool> events = std::make_shared<EventPool>();
     bool ordered_valid = false;
     uint64_t* d_tbl[3] = {nullptr, nullptr, nullptr};   // dispatch, combine, consumer pointer tables
     std::vector<uint64_t> tbl_cache[3];                  // what the device tables hold
@@ -172,6 +208,7 @@ struct mc_ep_world {
         for (void* p : retired) (void)hipFree(p);
         if (comm_stream) (void)hipStreamDestroy(comm_stream);
         if (ordered) (void)hipEventDestroy(ordered);
+        if (fence) (void)hipEventDestroy(fence);
         if (switched) (void)hipSetDevice(prev);
     }
 };
@@ -613,15 +650,17 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     return MC_EP_OK;
 }
 
-// Streams of a round: run on the callers' stream when they all share one and
-// nobody asked for an event (the reference's hook mode launches there too,
-// mooncake_ep_buffer.cpp:225); otherwise on the world's communication stream,
-// fenced against every caller's stream before and after, as the reference's
-// default mode does (:227, :325-327).
+// Streams of a round.  When every caller of the round is on one stream, the round runs there: an
+// async_finish caller still gets its event (recorded behind the round's kernels), a hook caller its
+// hook, and nothing has to cross streams - on one GPU there is no link transfer for later work of that
+// stream to overlap with, while every cross-stream hand-off costs about 10 us of device time.  With
+// callers on different streams, or with the option "comm_stream" set, the round runs on the world's
+// communication stream, fenced against every caller's stream before and after, which is the reference's
+// arrangement (mooncake_ep_buffer.cpp:225-227, :318-327).
 template <typename Post>
 hipStream_t pick_launch_stream(mc_ep_world* w, const std::vector<Post>& posts, bool* shared) {
     hipStream_t first = nullptr;
-    bool have = false, same = true, any_async = false;
+    bool have = false, same = true;
     for (const auto& p : posts) {
         if (!p.present) continue;
         if (!have) {
@@ -630,9 +669,8 @@ hipStream_t pick_launch_stream(mc_ep_world* w, const std::vector<Post>& posts, b
         } else if (p.stream != first) {
             same = false;
         }
-        any_async |= p.async;
     }
-    *shared = have && same && !any_async;
+    *shared = have && same && w->tuning.comm_stream == 0;
     return *shared ? first : w->comm_stream;
 }
 
@@ -645,31 +683,30 @@ int fence_before(mc_ep_world* w, const std::vector<Post>& posts, hipStream_t lau
         for (auto s : seen) dup |= (s == p.stream);
         if (dup) continue;
         seen.push_back(p.stream);
-        hipEvent_t ev;
-        MC_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
-        hipError_t e1 = hipEventRecord(ev, p.stream);
-        hipError_t e2 = (e1 == hipSuccess) ? hipStreamWaitEvent(launch, ev, 0) : e1;
-        (void)hipEventDestroy(ev);
-        MC_HIP(e2);
+        // a wait refers to what the event held when the wait was issued, so one event serves every stream
+        MC_HIP(hipEventRecord(w->fence, p.stream));
+        MC_HIP(hipStreamWaitEvent(launch, w->fence, 0));
     }
-    (void)w;
     return MC_EP_OK;
 }
 
 template <typename Post>
-int fence_after(const std::vector<Post>& posts, hipStream_t launch, Round* round) {
-    MC_HIP(hipEventCreateWithFlags(&round->done, hipEventDisableTiming));
-    MC_HIP(hipEventRecord(round->done, launch));
-    std::vector<hipStream_t> seen;
+int fence_after(mc_ep_world* w, const std::vector<Post>& posts, hipStream_t launch, Round* round) {
+    round->waited.assign(1, launch);      // work queued on the launch stream is behind the round anyway
+    // the completion event is recorded only when somebody can ask for it: an async caller's
+    // EventHandle, or a caller on another stream (a record costs a few us of device time)
+    bool needed = false;
+    for (const auto& p : posts) needed |= p.present && (p.async || p.stream != launch);
+    if (needed) {
+        round->pool = w->events;
+        if (int e = round->pool->take(&round->done)) return e;
+        MC_HIP(hipEventRecord(round->done, launch));
+    }
     for (const auto& p : posts) {
         // default mode: the caller's stream waits for the result; async and
         // hook callers wait through their event / hook
-        if (!p.present || p.async || p.hook || p.stream == launch) continue;
-        bool dup = false;
-        for (auto s : seen) dup |= (s == p.stream);
-        if (dup) continue;
-        seen.push_back(p.stream);
-        MC_HIP(hipStreamWaitEvent(p.stream, round->done, 0));
+        if (!p.present || p.async || p.hook) continue;
+        if (int e = round->make_wait(p.stream)) return e;
     }
     round->launched = true;
     return MC_EP_OK;
@@ -730,15 +767,21 @@ int launch_dispatch_round(mc_ep_world* w, PendingRound<DispatchPost>& pr) {
         return e;
     Round* round = pr.state.get();
     round->launch_stream = launch;
-    if (!two_part) return fence_after(pr.posts, launch, round);
-    MC_HIP(hipEventCreateWithFlags(&round->done, hipEventDisableTiming));
+    if (!two_part) return fence_after(w, pr.posts, launch, round);
+    bool needed = false;
+    for (const auto& p : pr.posts) needed |= p.present && p.stream != launch;
+    if (needed) {
+        round->pool = w->events;
+        if (int e = round->pool->take(&round->done)) return e;
+    }
     round->finish = [=]() -> int {
         DeviceGuard g(w->device);
         if (int e = world_dispatch_impl(w, x.data(), idx.data(), nt.data(), hidden, num_topk, max_tokens, num_experts,
                                         use_fp8, rx.data(), rs.data(), rc.data(), si.data(), lr.data(),
                                         MC_EP_PHASE_FINISH, launch))
             return e;
-        MC_HIP(hipEventRecord(round->done, launch));
+        if (round->done) MC_HIP(hipEventRecord(round->done, launch));
+        round->waited.assign(1, launch);
         return MC_EP_OK;
     };
     w->unfinished = pr.state;
@@ -775,7 +818,7 @@ int launch_combine_round(mc_ep_world* w, PendingRound<CombinePost>& pr) {
                                    out.data(), MC_EP_PHASE_ALL, launch))
         return e;
     pr.state->launch_stream = launch;
-    return fence_after(pr.posts, launch, pr.state.get());
+    return fence_after(w, pr.posts, launch, pr.state.get());
 }
 
 template <typename Post>
@@ -880,6 +923,7 @@ int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
     }
     MC_HIP(hipStreamCreateWithFlags(&w->comm_stream, hipStreamNonBlocking));
     MC_HIP(hipEventCreateWithFlags(&w->ordered, hipEventDisableTiming));
+    MC_HIP(hipEventCreateWithFlags(&w->fence, hipEventDisableTiming));
     for (int i = 0; i < 3; ++i) {
         const int fields[3] = {(int)DF_COUNT, (int)CF_COUNT, (int)XF_COUNT};
         const size_t words = (size_t)fields[i] * num_ranks;
@@ -924,6 +968,7 @@ static int* option_slot(Tuning& t, const char* name) {
     if (!strcmp(name, "pack_nt")) return &t.pack_nt;
     if (!strcmp(name, "uniform")) return &t.uniform;
     if (!strcmp(name, "fp8_arith")) return &t.fp8_arith;
+    if (!strcmp(name, "comm_stream")) return &t.comm_stream;
     if (!strcmp(name, "combine_direct")) return &t.combine_direct;
     if (!strcmp(name, "combine_chunks")) return &t.combine_chunks;
     if (!strcmp(name, "routing_sum")) return &t.routing_sum;
@@ -1304,8 +1349,7 @@ int mc_ep_event_current_stream_wait(mc_ep_event_t* ev, uint64_t stream_ptr) {
         return MC_EP_OK;
     }
     if (!ev->round || !ev->round->launched) return round_not_ready(ev->round.get());
-    MC_HIP(hipStreamWaitEvent((hipStream_t)stream_ptr, ev->round->done, 0));
-    return MC_EP_OK;
+    return ev->round->make_wait((hipStream_t)stream_ptr);
 }
 
 int mc_ep_event_synchronize(mc_ep_event_t* ev) {
@@ -1334,8 +1378,7 @@ int mc_ep_hook_call(mc_ep_hook_t* h) {
     if (h->round->finish)
         if (int e = finish_round(h->world, h->round.get())) return e;
     if (!h->round->failure.empty()) return round_not_ready(h->round.get());
-    if (h->stream != h->round->launch_stream) MC_HIP(hipStreamWaitEvent(h->stream, h->round->done, 0));
-    return MC_EP_OK;
+    return h->round->make_wait(h->stream);
 }
 
 int mc_ep_hook_destroy(mc_ep_hook_t* h) {

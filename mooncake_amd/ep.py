@@ -3,6 +3,13 @@
 `Buffer`, `EventHandle`, `get_ep_buffer_size_hint`, `MAX_QP_COUNT`, with the
 bound names and argument order of the reference, on top of the C ABI.
 
+Two bindings of the same C ABI exist.  The compiled one, `mooncake_amd._ep`
+(pybind11, csrc/ep_py.cpp - what the reference's own module is), is the one
+used; `MOONCAKE_AMD_EP_BINDING=ctypes` selects the ctypes binding in this file
+instead (a build without a host compiler).  `BINDING` names the one in use.
+Either way every call ends in libmooncake_ep_hip.so: there is no other
+implementation behind this module.
+
 One GPU holds the whole expert-parallel world: Buffers created with the same
 `World` (or, by default, with the same `num_ranks` in this process) are the
 logical ranks of one world.
@@ -10,12 +17,25 @@ logical ranks of one world.
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_void_p
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 from . import _lib
 
 MAX_QP_COUNT = 256   # mooncake_ep_configs.cuh:5
+
+_native = None
+if os.environ.get("MOONCAKE_AMD_EP_BINDING", "pybind11") != "ctypes":
+    try:
+        from . import _ep as _native
+    except ImportError as exc:
+        raise ImportError(
+            "mooncake_amd._ep (the compiled Python module) is not built; run "
+            f"`make -C {os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc')}` "
+            "or set MOONCAKE_AMD_EP_BINDING=ctypes") from exc
+    assert _native.MAX_QP_COUNT == MAX_QP_COUNT
+BINDING = "pybind11" if _native is not None else "ctypes"
 
 
 def get_ep_buffer_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
@@ -28,13 +48,23 @@ class World:
     """R logical EP ranks resident in the current device's HBM."""
 
     def __init__(self, num_ranks: int):
-        handle = c_void_p()
-        _lib.check(_lib.lib().mc_ep_world_create(int(num_ranks), ctypes.byref(handle)))
-        self._h = handle
+        _lib.lib()                       # the HIP library itself must load, whichever binding is used
+        if _native is not None:
+            # the compiled module owns the world (its Buffers, events and hooks keep it alive)
+            self._native = _native.World(int(num_ranks))
+            self._h = c_void_p(self._native.handle)
+        else:
+            self._native = None
+            handle = c_void_p()
+            _lib.check(_lib.lib().mc_ep_world_create(int(num_ranks), ctypes.byref(handle)))
+            self._h = handle
         self.num_ranks = int(num_ranks)
 
     def close(self) -> None:
-        if self._h:
+        if self._native is not None:
+            self._native = None          # destroyed when the last Buffer / event / hook of the world goes
+            self._h = None
+        elif self._h:
             _lib.lib().mc_ep_world_destroy(self._h)
             self._h = None
 
@@ -62,6 +92,14 @@ class World:
     def prepare_dispatch(self, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk,
                          num_max_dispatch_tokens_per_rank, num_experts, use_fp8, recv_x_ptrs, recv_scales_ptrs,
                          recv_count_ptrs, src_info_ptrs, layout_range_ptrs):
+        if self._native is not None:
+            return self._native.prepare_dispatch(
+                [int(v) for v in x_ptrs], [int(v) for v in topk_idx_ptrs], [int(v) for v in num_tokens], hidden,
+                num_topk, num_max_dispatch_tokens_per_rank, num_experts, bool(use_fp8),
+                [int(v) for v in recv_x_ptrs],
+                [int(v) for v in recv_scales_ptrs] if (use_fp8 and recv_scales_ptrs is not None) else None,
+                [int(v) for v in recv_count_ptrs], [int(v) for v in src_info_ptrs],
+                [int(v) for v in layout_range_ptrs])
         u = _lib.u64_array
         fn = _lib.lib().mc_ep_world_dispatch
         args = (self._h, u(x_ptrs), u(topk_idx_ptrs), _lib.i32_array(num_tokens), hidden, num_topk,
@@ -90,6 +128,12 @@ class World:
     def prepare_combine(self, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
                         active_ranks_ptrs, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
                         num_experts, combined_x_ptrs):
+        if self._native is not None:
+            ints = lambda vs: [int(v) for v in vs]
+            return self._native.prepare_combine(
+                ints(x_ptrs), None, 0, False, ints(topk_idx_ptrs), ints(topk_weights_ptrs), ints(src_info_ptrs),
+                ints(layout_range_ptrs), ints(active_ranks_ptrs), ints(num_combined_tokens), hidden, num_topk,
+                num_max_dispatch_tokens_per_rank, num_experts, ints(combined_x_ptrs))
         u = _lib.u64_array
         fn = _lib.lib().mc_ep_world_combine
         args = (self._h, u(x_ptrs), u(topk_idx_ptrs), u(topk_weights_ptrs), u(src_info_ptrs), u(layout_range_ptrs),
@@ -108,6 +152,13 @@ class World:
                                combined_x_ptrs):
         """Combine straight from dispatch's packed output (fp8 payload with scales, or bf16 when
         recv_scales_ptrs is None) times expert_factor[expert] (0: none): cast_back + combine in one."""
+        if self._native is not None:
+            ints = lambda vs: [int(v) for v in vs]
+            return self._native.prepare_combine(
+                ints(recv_x_ptrs), ints(recv_scales_ptrs) if recv_scales_ptrs is not None else None,
+                int(expert_factor_ptr), True, ints(topk_idx_ptrs), ints(topk_weights_ptrs), ints(src_info_ptrs),
+                ints(layout_range_ptrs), ints(active_ranks_ptrs), ints(num_combined_tokens), hidden, num_topk,
+                num_max_dispatch_tokens_per_rank, num_experts, ints(combined_x_ptrs))
         u = _lib.u64_array
         fn = _lib.lib().mc_ep_world_combine_packed
         args = (self._h, u(recv_x_ptrs), u(recv_scales_ptrs) if recv_scales_ptrs is not None else None,
@@ -183,8 +234,8 @@ def default_world(num_ranks: int) -> World:
     return w
 
 
-class EventHandle:
-    """mooncake_ep_event.h:9-42."""
+class _CtypesEventHandle:
+    """mooncake_ep_event.h:9-42 (ctypes binding)."""
 
     def __init__(self, stream_ptr: int = 0, _handle: Optional[c_void_p] = None):
         if _handle is not None:
@@ -225,8 +276,8 @@ class _RecvHook:
             pass
 
 
-class Buffer:
-    """One logical rank's MooncakeEpBuffer (ep_py.cpp:26-46)."""
+class _CtypesBuffer:
+    """One logical rank's MooncakeEpBuffer (ep_py.cpp:26-46), ctypes binding."""
 
     def __init__(self, rank: int, num_ranks: int, num_ep_buffer_bytes: int, disable_p2p: bool = False,
                  world: Optional[World] = None):
@@ -298,7 +349,7 @@ class Buffer:
                  use_fp8: bool, packed_recv_x_ptr: int, packed_recv_x_scales_ptr: int, packed_recv_count_ptr: int,
                  packed_recv_src_info_ptr: int, packed_recv_layout_range_ptr: int, async_: bool,
                  return_recv_hook: bool, compute_stream_ptr: int
-                 ) -> Tuple[Optional[EventHandle], Optional[Callable[[], None]]]:
+                 ) -> Tuple[Optional[object], Optional[Callable[[], None]]]:
         ev, hook = c_void_p(), c_void_p()
         _lib.check(_lib.lib().mc_ep_buffer_dispatch(
             self._h, x_ptr, topk_idx_ptr, active_ranks_ptr, num_tokens, hidden, num_topk,
@@ -306,17 +357,42 @@ class Buffer:
             packed_recv_x_scales_ptr, packed_recv_count_ptr, packed_recv_src_info_ptr,
             packed_recv_layout_range_ptr, int(bool(async_)), int(bool(return_recv_hook)), compute_stream_ptr,
             ctypes.byref(ev), ctypes.byref(hook)))
-        return (EventHandle(_handle=ev) if ev else None, _RecvHook(hook) if hook else None)
+        return (_CtypesEventHandle(_handle=ev) if ev else None, _RecvHook(hook) if hook else None)
 
     def combine(self, x_ptr: int, topk_idx_ptr: int, topk_weights_ptr: int, src_info_ptr: int,
                 layout_range_ptr: int, active_ranks_ptr: int, num_local_experts: int, num_combined_tokens: int,
                 hidden: int, num_topk: int, num_max_dispatch_tokens_per_rank: int, num_experts: int,
                 timeout_us: int, zero_copy: bool, combined_x_ptr: int, async_: bool, return_recv_hook: bool,
-                compute_stream_ptr: int) -> Tuple[Optional[EventHandle], Optional[Callable[[], None]]]:
+                compute_stream_ptr: int) -> Tuple[Optional[object], Optional[Callable[[], None]]]:
         ev, hook = c_void_p(), c_void_p()
         _lib.check(_lib.lib().mc_ep_buffer_combine(
             self._h, x_ptr, topk_idx_ptr, topk_weights_ptr, src_info_ptr, layout_range_ptr, active_ranks_ptr,
             num_local_experts, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
             num_experts, timeout_us, int(bool(zero_copy)), combined_x_ptr, int(bool(async_)),
             int(bool(return_recv_hook)), compute_stream_ptr, ctypes.byref(ev), ctypes.byref(hook)))
-        return (EventHandle(_handle=ev) if ev else None, _RecvHook(hook) if hook else None)
+        return (_CtypesEventHandle(_handle=ev) if ev else None, _RecvHook(hook) if hook else None)
+
+
+if _native is not None:
+    EventHandle = _native.EventHandle
+
+    class Buffer(_native.Buffer):
+        """One logical rank's MooncakeEpBuffer (ep_py.cpp:26-46): the compiled module's class, which takes
+        the world it belongs to as this package's `World`."""
+
+        def __init__(self, rank: int, num_ranks: int, num_ep_buffer_bytes: int, disable_p2p: bool = False,
+                     world: Optional[World] = None):
+            w = world if world is not None else default_world(num_ranks)
+            if w.num_ranks != num_ranks:
+                raise RuntimeError(f"world has {w.num_ranks} ranks, Buffer asked for {num_ranks}")
+            _native.Buffer.__init__(self, int(rank), int(num_ranks), int(num_ep_buffer_bytes), bool(disable_p2p),
+                                    w._native)
+            self._world = w
+
+    _benchmark_legacy_buffer = _native._benchmark_legacy_buffer
+    _LegacyBufferPerfTensors = _native._LegacyBufferPerfTensors
+    _LegacyBufferPerfConfig = _native._LegacyBufferPerfConfig
+    _LegacyBufferPerfResult = _native._LegacyBufferPerfResult
+else:
+    EventHandle = _CtypesEventHandle
+    Buffer = _CtypesBuffer

@@ -66,3 +66,31 @@ def test_header_is_plain_c_and_structs_match_ctypes(tmp_path):
     assert sizes == [ctypes.sizeof(_lib.LegacyPerfTensors), ctypes.sizeof(_lib.LegacyPerfConfig),
                      _lib.LegacyPerfConfig.compute_stream_ptr.offset, ctypes.sizeof(_lib.LegacyPerfResult),
                      _lib.LegacyPerfTensors.combined_x_ptrs.offset]
+
+
+def test_compiled_module_binds_what_the_reference_module_binds():
+    """mooncake_amd._ep is the compiled counterpart of mooncake._ep (mooncake-ep/src/ep_py.cpp:14-46): the same
+    module-level names, the same methods on Buffer and EventHandle, the legacy benchmark's three structs with the
+    reference's field names (legacy_buffer_perf.cpp:151-199).  Importing it needs no GPU."""
+    from mooncake_amd import _ep, ep
+    assert ep.BINDING == "pybind11" and ep.Buffer.__mro__[1] is _ep.Buffer and ep.EventHandle is _ep.EventHandle
+    for name in ("get_ep_buffer_size_hint", "EventHandle", "MAX_QP_COUNT", "Buffer", "_benchmark_legacy_buffer",
+                 "_LegacyBufferPerfTensors", "_LegacyBufferPerfConfig", "_LegacyBufferPerfResult"):
+        assert hasattr(_ep, name), name
+    for method in ("ibgda_disabled", "p2p_enabled", "use_fast_path", "update_local_qpns", "is_roce", "sync_ibgda_peers",
+                   "get_mr_info", "get_gid", "get_local_qpns", "get_local_lids", "get_ipc_handle",
+                   "sync_nvlink_ipc_handles", "dispatch", "combine"):
+        assert callable(getattr(_ep.Buffer, method)), method
+    for method in ("current_stream_wait", "synchronize"):
+        assert callable(getattr(_ep.EventHandle, method)), method
+    t, c = _ep._LegacyBufferPerfTensors(), _ep._LegacyBufferPerfConfig()
+    for field in ("x_ptr", "topk_idx_ptr", "topk_weights_ptr", "active_ranks_ptr", "expert_x_ptr", "packed_recv_x_ptr",
+                  "packed_recv_count_ptr", "packed_recv_src_info_ptr", "packed_recv_layout_range_ptr", "combined_x_ptr"):
+        assert getattr(t, field) == []
+    assert (c.timeout_us, c.warmups, c.iterations, c.compute_stream_ptr) == (-1, 20, 30, 0)
+    assert _ep.MAX_QP_COUNT == 256 and _ep.get_ep_buffer_size_hint(128, 7168, 32, 256) == 1883246592
+    # the constructor's signature: (rank, num_ranks, num_ep_buffer_bytes, disable_p2p=False[, world])
+    import re
+    sig = _ep.Buffer.__init__.__doc__
+    assert re.findall(r"(\w+): ", sig) == ["self", "rank", "num_ranks", "num_ep_buffer_bytes", "disable_p2p", "world"]
+    assert "disable_p2p: bool = False" in sig

@@ -52,10 +52,13 @@ MODES = [(False, False), (True, False), (False, True)]      # (async_finish, ret
 @pytest.mark.parametrize("use_fp8", [False, True], ids=["bf16", "fp8"])
 @pytest.mark.parametrize("async_finish,return_recv_hook", MODES, ids=["default", "async", "hook"])
 @pytest.mark.parametrize("fail_rank", [-1, 2], ids=["all_alive", "rank2_dead"])
-def test_grid_closed_form(gpu_device, oracle, use_fp8, async_finish, return_recv_hook, fail_rank):
+@pytest.mark.parametrize("comm_stream", [0, 1], ids=["callers_stream", "comm_stream"])
+def test_grid_closed_form(gpu_device, oracle, use_fp8, async_finish, return_recv_hook, fail_rank, comm_stream):
     num_ranks, max_tokens, hidden, num_experts, top_k = 4, 256, 2048, 288, 8
-    announce(f"grid fp8={use_fp8} async={async_finish} hook={return_recv_hook} fail_rank={fail_rank}")
+    announce(f"grid fp8={use_fp8} async={async_finish} hook={return_recv_hook} fail_rank={fail_rank} "
+             f"comm_stream={comm_stream}")
     world, bufs = make_world(num_ranks, max_tokens, hidden, num_experts)
+    world.set_option("comm_stream", comm_stream)     # 1: the reference's arrangement, rounds on a stream of their own
     L = num_experts // num_ranks
     alive = [r for r in range(num_ranks) if r != fail_rank]
     timeout_us = 5_000_000 if fail_rank != -1 else -1
