@@ -30,6 +30,7 @@ extern "C" {
 #define MC_EP_ERR_HIP 2         /* a HIP runtime call failed */
 #define MC_EP_ERR_PENDING 3     /* a collective is waited on before every live rank has called it */
 #define MC_EP_ERR_UNSUPPORTED 4 /* zero-copy combine etc. (NotImplementedError in the reference) */
+#define MC_EP_ERR_INVALID 5     /* std::invalid_argument in the reference (ValueError through pybind11) */
 
 /* mooncake_ep_configs.cuh:5 */
 #define MC_EP_MAX_QP_COUNT 256

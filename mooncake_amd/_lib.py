@@ -12,7 +12,7 @@ from ctypes import POINTER, Structure, c_char_p, c_double, c_int, c_int32, c_int
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmooncake_ep_hip.so")
 
-OK, ERR_ASSERT, ERR_HIP, ERR_PENDING, ERR_UNSUPPORTED = 0, 1, 2, 3, 4
+OK, ERR_ASSERT, ERR_HIP, ERR_PENDING, ERR_UNSUPPORTED, ERR_INVALID = 0, 1, 2, 3, 4, 5
 PHASE_LAYOUT, PHASE_DATA, PHASE_FINISH, PHASE_ALL = 1, 2, 4, 7
 
 _lib = None
@@ -111,12 +111,15 @@ def last_error() -> str:
 def check(rc: int) -> None:
     """Map an MC_EP_ERR_* code to the exception the reference raises: host
     assertions and HIP failures become RuntimeError (EPException through
-    pybind11), unsupported features NotImplementedError."""
+    pybind11), unsupported features NotImplementedError, what the reference
+    rejects with std::invalid_argument ValueError."""
     if rc == OK:
         return
     msg = last_error()
     if rc == ERR_UNSUPPORTED:
         raise NotImplementedError(msg)
+    if rc == ERR_INVALID:
+        raise ValueError(msg)          # std::invalid_argument through pybind11
     raise RuntimeError(msg)
 
 

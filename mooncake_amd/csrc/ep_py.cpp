@@ -39,6 +39,7 @@ void check(int rc) {
         PyErr_SetString(PyExc_NotImplementedError, msg ? msg : "unsupported");
         throw py::error_already_set();
     }
+    if (rc == MC_EP_ERR_INVALID) throw std::invalid_argument(msg ? msg : "invalid argument");   // ValueError
     throw std::runtime_error(msg ? msg : "mooncake_ep_hip: unknown failure");
 }
 

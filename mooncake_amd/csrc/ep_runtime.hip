@@ -1091,7 +1091,7 @@ int mc_ep_world_legacy_buffer_perf(mc_ep_world_t* w, const mc_ep_legacy_perf_ten
     if (c->num_tokens <= 0 || c->hidden <= 0 || c->num_topk <= 0 ||
         c->num_max_dispatch_tokens_per_rank < c->num_tokens || c->num_experts <= 0 || c->num_local_experts <= 0 ||
         c->warmups < 0 || c->iterations <= 1)
-        return fail(MC_EP_ERR_ASSERT, "invalid legacy EP benchmark configuration");
+        return fail(MC_EP_ERR_INVALID, "invalid legacy EP benchmark configuration");
     const uint64_t* const fields[] = {t->x_ptrs,
                                       t->topk_idx_ptrs,
                                       t->topk_weights_ptrs,
@@ -1103,9 +1103,9 @@ int mc_ep_world_legacy_buffer_perf(mc_ep_world_t* w, const mc_ep_legacy_perf_ten
                                       t->packed_recv_layout_range_ptrs,
                                       t->combined_x_ptrs};
     for (const uint64_t* f : fields) {
-        if (f == nullptr) return fail(MC_EP_ERR_ASSERT, "legacy EP benchmark received a null tensor pointer");
+        if (f == nullptr) return fail(MC_EP_ERR_INVALID, "legacy EP benchmark received a null tensor pointer");
         for (int r = 0; r < w->R; ++r)
-            if (f[r] == 0) return fail(MC_EP_ERR_ASSERT, "legacy EP benchmark received a null tensor pointer");
+            if (f[r] == 0) return fail(MC_EP_ERR_INVALID, "legacy EP benchmark received a null tensor pointer");
     }
     MC_ASSERT(c->num_local_experts * w->R == c->num_experts);
 

@@ -207,6 +207,19 @@ class World:
         world: returns (average_us, min_us, max_us) of recv_count clear + bf16
         dispatch + combine.  `tensors` maps the field names of
         LegacyBufferPerfTensors (x_ptr -> "x", ...) to per-rank addresses."""
+        if self._native is not None:
+            # the compiled module's binding of the loop, as the reference's script calls it
+            # (mooncake-ep/benchmarks/legacy_buffer_perf.py:84-107)
+            nt, nc = _native._LegacyBufferPerfTensors(), _native._LegacyBufferPerfConfig()
+            for field, _ in _lib.LegacyPerfTensors._fields_:
+                values = tensors.get(field[:-len("_ptrs")])
+                setattr(nt, field[:-1], [int(v) for v in values] if values is not None else [])
+            nc.num_tokens, nc.hidden, nc.num_topk, nc.num_local_experts = num_tokens, hidden, num_topk, num_local_experts
+            nc.num_max_dispatch_tokens_per_rank, nc.num_experts = num_max_dispatch_tokens_per_rank, num_experts
+            nc.timeout_us, nc.warmups, nc.iterations = timeout_us, warmups, iterations
+            nc.compute_stream_ptr = int(compute_stream_ptr)
+            res = _native._benchmark_legacy_buffer(self._native, nt, nc)
+            return res.average_us, res.min_us, res.max_us
         t = _lib.LegacyPerfTensors()
         keep = []
         for field, _ in _lib.LegacyPerfTensors._fields_:

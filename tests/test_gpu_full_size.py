@@ -79,3 +79,57 @@ def test_named_config_full_size(gpu_device, oracle, name, summed):
     eo.view(R * L, RM, cfg.hidden)[mask] = rows
     want = oracle.combine(eo, idx, data["topk_weights"], ref["src_info"], ref["layout_range"], nt, cfg.max_tokens, E)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_dsv3_decode_full_size_through_the_per_rank_buffer_api(gpu_device, oracle):
+    """The headline world driven the way the reference's callers drive it: 32 `Buffer.dispatch` and 32
+    `Buffer.combine` calls (the Python wrapper with the reference's signature, async_finish), every rank's
+    outputs against the oracle bit for bit."""
+    from mooncake_amd import Buffer, LogicalGroup
+    cfg = CONFIGS["dsv3_decode"]
+    announce(f"full size through Buffer.dispatch / Buffer.combine {cfg}")
+    data = generate(cfg, seed=0)
+    R, T, E, L, H = cfg.num_ranks, cfg.tokens_per_rank, cfg.num_experts, cfg.num_local_experts, cfg.hidden
+    world, groups = LogicalGroup.make_world(R)
+    nbytes = Buffer.get_ep_buffer_size_hint(cfg.max_tokens, H, R, E)
+    bufs = [Buffer(g, nbytes) for g in groups]
+    x = data["x"].to(gpu_device)
+    idx = data["topk_idx"].to(gpu_device)
+    w = data["topk_weights"].to(gpu_device)
+    disp = [bufs[r].dispatch(x[r], idx[r], None, cfg.max_tokens, E, -1, use_fp8=True, async_finish=True)
+            for r in range(R)]
+    for d in disp:
+        d[3].current_stream_wait()
+    torch.cuda.synchronize()
+    nt = [T] * R
+    ref = oracle.dispatch(data["x"], data["topk_idx"], nt, cfg.max_tokens, E, True, poison=None)
+    RM = R * cfg.max_tokens
+    for r in range(R):
+        (recv_x, scales), cnt, handle, _, _ = disp[r]
+        cnt_cpu = cnt.cpu()
+        assert torch.equal(cnt_cpu, ref["recv_count"][r])
+        assert torch.equal(handle[1].cpu(), ref["layout_range"][r])
+        assert scales.shape == (L, RM, H // 128) and scales.stride() == (H // 128 * RM, 1, RM)
+        mask = torch.arange(RM).view(1, RM) < cnt_cpu.view(L, 1)
+        assert torch.equal(handle[0].cpu()[mask], ref["src_info"][r][mask])
+        assert torch.equal(recv_x.view(torch.uint8).cpu()[mask], ref["recv_x"][r].view(torch.uint8)[mask])
+        assert torch.equal(scales.cpu()[mask].contiguous().view(torch.int32),
+                           ref["scales"][r][mask].contiguous().view(torch.int32))
+    # the mock expert of the reference's grid test, then combine
+    factor = torch.arange(E, dtype=torch.float32) * 0.1 + 1.0
+    rows = oracle.cast_back(ref["recv_x"], ref["scales"], ref["recv_count"], factor)
+    want = oracle.combine(rows, data["topk_idx"], data["topk_weights"], ref["src_info"], ref["layout_range"], nt,
+                          cfg.max_tokens, E)
+    outs = []
+    for r in range(R):
+        (recv_x, scales), cnt, handle, _, _ = disp[r]
+        f = factor[r * L:(r + 1) * L].to(gpu_device).view(L, 1, 1)
+        once = (recv_x.float().view(L, RM, H // 128, 128) * scales.unsqueeze(-1)).view(L, RM, H).to(torch.bfloat16)
+        expert_out = (once.float() * f).to(torch.bfloat16)
+        outs.append(bufs[r].combine(expert_out, idx[r], w[r], None, -1, handle, async_finish=True))
+        del once, expert_out
+    for o in outs:
+        o[1].current_stream_wait()
+    torch.cuda.synchronize()
+    for r in range(R):
+        assert torch.equal(outs[r][0].cpu().view(torch.int16), want[r].view(torch.int16)), f"rank {r}"

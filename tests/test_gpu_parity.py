@@ -16,6 +16,18 @@ SMALL = [
     EPConfig("tiny_fp8", 2, 4, 128, 4, 2, True),
     EPConfig("odd_hidden_fp8", 4, 24, 2560, 16, 3, True),            # 2.5 slabs of 1024
     EPConfig("odd_hidden_bf16", 4, 24, 2560, 16, 3, False),
+    # the hidden sizes the reference instantiates its kernels for (SWITCH_HIDDEN, mooncake_ep_launch.cuh:66-87)
+    # beyond the ones other cases use: 1024-element pack slabs and 512-element combine slabs with and without a tail
+    EPConfig("h3072_fp8", 4, 20, 3072, 16, 4, True),
+    EPConfig("h3072_bf16", 4, 20, 3072, 16, 4, False),
+    EPConfig("h5120_fp8", 4, 20, 5120, 32, 6, True),
+    EPConfig("h5120_bf16", 4, 20, 5120, 32, 6, False),
+    EPConfig("h6144_fp8", 2, 36, 6144, 16, 8, True),
+    EPConfig("h6144_bf16", 2, 36, 6144, 16, 8, False),
+    EPConfig("h8192_fp8", 4, 24, 8192, 32, 8, True),
+    EPConfig("h8192_bf16", 4, 24, 8192, 32, 8, False),
+    EPConfig("h4096_fp8", 4, 24, 4096, 32, 8, True),
+    EPConfig("h7168_bf16", 4, 24, 7168, 32, 8, False),
     EPConfig("k11", 4, 40, 2048, 32, 11, True),                      # the reference's top-k cap
     EPConfig("k16_bf16", 2, 20, 1024, 32, 16, False),
     EPConfig("one_rank", 1, 36, 1024, 6, 2, True),                   # group_size == 1
@@ -159,6 +171,10 @@ def test_duplicate_experts_follow_the_oracle(gpu_device, oracle):
 COMBINE_CASES = [
     EPConfig("tiny_c", 2, 4, 128, 4, 2, False),
     EPConfig("odd_hidden_c", 4, 24, 2560, 16, 3, False),
+    EPConfig("h3072_c", 4, 20, 3072, 16, 4, False),
+    EPConfig("h5120_c", 4, 20, 5120, 32, 6, True),
+    EPConfig("h6144_c", 2, 36, 6144, 16, 8, False),
+    EPConfig("h8192_c", 4, 24, 8192, 32, 8, True),
     EPConfig("k11_c", 4, 40, 2048, 32, 11, False),
     EPConfig("k16_c", 2, 20, 1024, 32, 16, False),
     EPConfig("masked_c", 8, 64, 1024, 8, 2, False, masked_fraction=0.3),
