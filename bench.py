@@ -60,6 +60,9 @@ def parse_args():
                     help="write this many MiB before every step of the per-kernel timing loop (cache flush)")
     ap.add_argument("--graph", action="store_true",
                     help="record the step into a HIP graph once and time replays instead of eager launches")
+    ap.add_argument("--stream-ceilings", action="store_true",
+                    help="instead of the workload, time synthetic streams with the data kernels' read : write mixes "
+                         "and byte counts (what the memory system gives each mix), and print them as JSON")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (the known-size "
                          "kernel that profiler FETCH_SIZE / WRITE_SIZE readings are scaled against)")
@@ -259,6 +262,38 @@ def time_python_buffer(h, steps, warmup):
     return {"us_per_step": round((time.perf_counter() - t0) / n * 1e6, 2), "steps": n}
 
 
+def stream_ceilings(cfg, S, iters):
+    """Synthetic streams (the library's stream_kernel: one 16-byte unit per thread, nothing else) with the read :
+    write mix and the byte counts of each data kernel of this workload, launched back to back."""
+    import torch
+    from mooncake_amd import _lib
+    lib = _lib.lib()
+    stream = int(torch.cuda.current_stream().cuda_stream)
+    H, N = cfg.hidden, cfg.total_tokens
+    unit = lambda nbytes: (int(nbytes) + 4095) // 4096 * 4096
+    out_rows, exp_rows = unit(N * H * 2), unit(S * H * 2)
+    fp8_rows = unit(S * H)
+    # name: (kind, unit_bytes, bytes read, bytes written)
+    mixes = {
+        "copy 1:1 (512 MiB each way)": (0, 512 << 20, 512 << 20, 512 << 20),
+        "read only (1 GiB)": (1, 1 << 30, 1 << 30, 0),
+        "write only (1 GiB)": (2, 1 << 30, 0, 1 << 30),
+        "widen 1:2, cast-back sized": (3, exp_rows, exp_rows // 2, exp_rows),
+        "gather 8:1, reduce sized": (4, out_rows, 8 * out_rows, out_rows),
+        "scatter 1:4, fp8-pack sized": (5, fp8_rows // 8, fp8_rows // 4, fp8_rows),
+    }
+    big = max(max(r, w) for _, _, r, w in mixes.values())
+    src = torch.empty(big, dtype=torch.uint8, device="cuda:0").fill_(3)
+    dst = torch.empty(big, dtype=torch.uint8, device="cuda:0")
+    res = {}
+    for name, (kind, ub, rd, wr) in mixes.items():
+        us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_stream(kind, dst.data_ptr(), src.data_ptr(), ub,
+                                                                          stream)), iters)
+        res[name] = {"us": round(us, 2), "read_MB": round(rd / 1e6, 1), "written_MB": round(wr / 1e6, 1),
+                     "GBps": round((rd + wr) / us / 1e3, 1), "pct_of_hbm_peak": round((rd + wr) / us / 1e3 / 80, 2)}
+    return res
+
+
 def cpu_baseline(cfg, data, bytes_total, budget_s):
     """The oracle (a scalar C restatement, OpenMP over tokens) timed on this
     host's cores on the same workload: whole steps until the budget is spent."""
@@ -315,6 +350,10 @@ def main():
     data = generate(cfg, seed=args.seed)
     S = int((data["topk_idx"] >= 0).sum())
     alg = algorithmic_bytes(cfg, S)
+
+    if args.stream_ceilings:
+        print(json.dumps({"workload": cfg.name, "stream_ceilings": stream_ceilings(cfg, S, args.kernel_iters)}))
+        return
 
     h = WorldHarness(cfg, device="cuda:0")
     opts = {}

@@ -285,12 +285,6 @@ int mc_ep_event_destroy(mc_ep_event_t* event);
 int mc_ep_hook_call(mc_ep_hook_t* hook);
 int mc_ep_hook_destroy(mc_ep_hook_t* hook);
 
-/* ---- measurement helper -------------------------------------------------- */
-
-/* Plain device copy of `bytes` (multiple of 16): the known-size kernel the
- * profiler's FETCH_SIZE / WRITE_SIZE readings are scaled against. */
-int mc_ep_debug_copy(uint64_t dst_ptr, uint64_t src_ptr, uint64_t bytes, uint64_t stream_ptr);
-
 #ifdef __cplusplus
 }
 #endif

@@ -83,7 +83,12 @@ SIGNATURES = {
     "mc_ep_event_destroy": (c_int, [c_void_p]),
     "mc_ep_hook_call": (c_int, [c_void_p]),
     "mc_ep_hook_destroy": (c_int, [c_void_p]),
+}
+
+# measurement helpers the library exports beside its public ABI (csrc/ep_debug.h)
+DEBUG_SIGNATURES = {
     "mc_ep_debug_copy": (c_int, [c_uint64, c_uint64, c_uint64, c_uint64]),
+    "mc_ep_debug_stream": (c_int, [c_int, c_uint64, c_uint64, c_uint64, c_uint64]),
 }
 
 
@@ -95,7 +100,7 @@ def lib() -> ctypes.CDLL:
                 f"{LIB_PATH} is not built; run `make -C {os.path.join(_HERE, 'csrc')}` "
                 "(the dispatch/combine path has no fallback without it)")
         handle = ctypes.CDLL(LIB_PATH)
-        for name, (restype, argtypes) in SIGNATURES.items():
+        for name, (restype, argtypes) in list(SIGNATURES.items()) + list(DEBUG_SIGNATURES.items()):
             fn = getattr(handle, name)
             fn.restype = restype
             fn.argtypes = argtypes

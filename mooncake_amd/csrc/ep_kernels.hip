@@ -337,6 +337,108 @@ __device__ __forceinline__ int summed_begin(const RoutingScratch& sc, const SelK
 }
 
 // ---------------------------------------------------------------------------
+// fp8 scales: from the pack waves' staging rows into the column-major output
+// ---------------------------------------------------------------------------
+// Staged scales -> column-major output.  A work item is 64 packed rows of one
+// expert times one part of kTransposeGroups scale groups, and a wave takes one
+// item: a lane learns its row's source token slot from row_src (left by the
+// pack waves), reads that token's scales as contiguous pieces, all in flight at
+// once, and stores them so that the wave writes 64 consecutive floats per scale
+// group.
+//
+// Which expert owns the wave's 64-row chunk follows from the per-expert row
+// counts alone: every wave scans ceil(count / 64) over the experts (a DPP scan
+// per 64 experts) and finds the expert whose chunk range holds its chunk
+// number.  The work list therefore holds no more items than there are chunks
+// (at most one partly filled chunk per expert), however uneven the routing is.
+constexpr int kTransposeGroups = 32;      // scale groups per wave: 128 bytes of staged scales per lane
+constexpr int kTransposeWaves = 4;        // waves per block of scale_transpose_kernel
+
+__device__ __forceinline__ void transpose_task(const uint64_t* __restrict__ tbl, const float* __restrict__ scale_stage,
+                                               const RoutingScratch& scratch, int R, int E, int G, int max_tokens,
+                                               int parts, int task) {
+    const int lane = wave_lane();
+    const int target = task / parts, part = task - target * parts;
+
+    // chunk ranges of the experts: expert e owns chunks [begin_e, begin_e + ceil(count_e / 64))
+    constexpr int kPre = 4;               // 64-expert pieces whose counts are loaded side by side
+    int pre_counts[kPre];
+#pragma unroll
+    for (int j = 0; j < kPre; ++j) {
+        const int ee = j * 64 + lane;
+        pre_counts[j] = 0;
+        if (ee < E) pre_counts[j] = scratch.counts[ee];
+    }
+    int carry = 0, e = -1, chunk = 0, count = 0;
+    auto piece = [&](int e0, int c) {
+        const int n = (c + 63) >> 6;
+        const int incl = wave_scan_inclusive(n);
+        const int begin = carry + incl - n;
+        const unsigned long long owns = __ballot(n > 0 && begin <= target && target < begin + n);
+        if (owns) {
+            const int l = __builtin_ctzll(owns);
+            e = e0 + l;
+            chunk = target - __builtin_amdgcn_readlane(begin, l);
+            count = __builtin_amdgcn_readlane(c, l);
+        }
+        carry += __builtin_amdgcn_readlane(incl, 63);
+    };
+#pragma unroll
+    for (int j = 0; j < kPre; ++j)
+        if (j * 64 < E) piece(j * 64, pre_counts[j]);
+    for (int e0 = kPre * 64; e0 < E; e0 += 64) {
+        const int ee = e0 + lane;
+        int c = 0;
+        if (ee < E) c = scratch.counts[ee];
+        piece(e0, c);
+    }
+    if (e < 0) return;                    // beyond the last chunk
+    e = __builtin_amdgcn_readfirstlane(e);
+    chunk = __builtin_amdgcn_readfirstlane(chunk);
+    count = __builtin_amdgcn_readfirstlane(count);
+
+    const int L = E / R, q = e / L, le = e - q * L;
+    const int64_t RM = (int64_t)R * max_tokens;
+    const int g0 = part * kTransposeGroups;
+    const int n = (g0 + kTransposeGroups < G ? g0 + kTransposeGroups : G) - g0;
+    const int row = chunk * 64 + lane;
+    const bool valid = row < count;
+    // the output address and the row's source slot, side by side
+    float* out = (float*)tbl[DF_RECV_SCALES * R + q];
+    int slot = 0;
+    if (valid) slot = scratch.row_src[(int64_t)e * RM + row];
+    const float* sp = scale_stage + (int64_t)slot * G + g0;
+    float* dp = out + ((int64_t)le * G + g0) * RM + row;
+    if ((G & 3) == 0) {
+        // 16-byte loads, all issued before the first store
+        constexpr int B = kTransposeGroups / 4;
+        float4 v[B];
+#pragma unroll
+        for (int j = 0; j < B; ++j) v[j] = (4 * j < n) ? *(const float4*)(sp + 4 * j) : make_float4(0, 0, 0, 0);
+        if (valid) {
+#pragma unroll
+            for (int j = 0; j < B; ++j) {
+                if (4 * j >= n) break;
+                dp[(int64_t)(4 * j + 0) * RM] = v[j].x;
+                dp[(int64_t)(4 * j + 1) * RM] = v[j].y;
+                dp[(int64_t)(4 * j + 2) * RM] = v[j].z;
+                dp[(int64_t)(4 * j + 3) * RM] = v[j].w;
+            }
+        }
+    } else if (valid) {
+        for (int g = 0; g < n; ++g) dp[(int64_t)g * RM] = sp[g];
+    }
+}
+
+__global__ __launch_bounds__(kTransposeWaves * 64) void scale_transpose_kernel(
+    const uint64_t* __restrict__ tbl, const float* __restrict__ scale_stage, RoutingScratch scratch, int R, int E,
+    int G, int max_tokens, int parts, int total_tasks) {
+    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * kTransposeWaves + (threadIdx.x >> 6));
+    if (task >= total_tasks) return;
+    transpose_task(tbl, scale_stage, scratch, R, E, G, max_tokens, parts, task);
+}
+
+// ---------------------------------------------------------------------------
 // dispatch pack
 // ---------------------------------------------------------------------------
 constexpr int kMaxPackWaves = 8;     // waves per block the launcher may choose
@@ -512,94 +614,6 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
 #pragma unroll
         for (int p = 0; p < 2; ++p)
             if (active[p]) store16<false>((void*)(row + off[p]), v[p]);
-    }
-}
-
-// Staged scales -> column-major output.  A work item is 64 packed rows of one
-// expert times one part of kTransposeGroups scale groups, and a wave takes one
-// item: a lane learns its row's source token slot from row_src (left by the
-// pack kernel), reads that token's scales as contiguous 16-byte pieces, all in
-// flight at once, and stores them so that the wave writes 64 consecutive floats
-// per scale group.
-//
-// Which expert owns the wave's 64-row chunk follows from the per-expert row
-// counts alone: every wave scans ceil(count / 64) over the experts (a few
-// shuffles per 64 experts) and finds the expert whose chunk range holds its
-// chunk number.  The grid therefore holds no more waves than there are chunks
-// (at most one partly filled chunk per expert), however uneven the routing is.
-constexpr int kTransposeGroups = 32;      // scale groups per wave: 8 loads of 16 bytes per lane
-constexpr int kTransposeWaves = 4;        // waves per block
-
-__global__ __launch_bounds__(kTransposeWaves * 64) void scale_transpose_kernel(
-    const uint64_t* __restrict__ tbl, const float* __restrict__ scale_stage, RoutingScratch scratch, int R, int E,
-    int G, int max_tokens, int parts, int total_tasks) {
-    const int lane = wave_lane();
-    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * kTransposeWaves + (threadIdx.x >> 6));
-    if (task >= total_tasks) return;
-    const int target = task / parts, part = task - target * parts;
-
-    // chunk ranges of the experts: expert e owns chunks [begin_e, begin_e + ceil(count_e / 64))
-    constexpr int kPre = 4;               // 64-expert pieces whose counts are loaded side by side
-    int pre_counts[kPre];
-#pragma unroll
-    for (int j = 0; j < kPre; ++j) {
-        const int ee = j * 64 + lane;
-        pre_counts[j] = (ee < E) ? scratch.counts[ee] : 0;
-    }
-    int carry = 0, e = -1, chunk = 0, count = 0;
-    auto piece = [&](int e0, int c) {
-        const int n = (c + 63) >> 6;
-        const int incl = wave_scan_inclusive(n);
-        const int begin = carry + incl - n;
-        const unsigned long long owns = __ballot(n > 0 && begin <= target && target < begin + n);
-        if (owns) {
-            const int l = __builtin_ctzll(owns);
-            e = e0 + l;
-            chunk = target - __builtin_amdgcn_readlane(begin, l);
-            count = __builtin_amdgcn_readlane(c, l);
-        }
-        carry += __builtin_amdgcn_readlane(incl, 63);
-    };
-#pragma unroll
-    for (int j = 0; j < kPre; ++j)
-        if (j * 64 < E) piece(j * 64, pre_counts[j]);
-    for (int e0 = kPre * 64; e0 < E; e0 += 64) {
-        const int ee = e0 + lane;
-        piece(e0, (ee < E) ? scratch.counts[ee] : 0);
-    }
-    if (e < 0) return;                    // beyond the last chunk
-    e = __builtin_amdgcn_readfirstlane(e);
-    chunk = __builtin_amdgcn_readfirstlane(chunk);
-    count = __builtin_amdgcn_readfirstlane(count);
-
-    const int L = E / R, q = e / L, le = e - q * L;
-    const int64_t RM = (int64_t)R * max_tokens;
-    const int g0 = part * kTransposeGroups;
-    const int n = (g0 + kTransposeGroups < G ? g0 + kTransposeGroups : G) - g0;
-    const int row = chunk * 64 + lane;
-    const bool valid = row < count;
-    // the output address and the row's source slot, side by side
-    float* out = (float*)tbl[DF_RECV_SCALES * R + q];
-    const int slot = valid ? scratch.row_src[(int64_t)e * RM + row] : 0;
-    const float* sp = scale_stage + (int64_t)slot * G + g0;
-    float* dp = out + ((int64_t)le * G + g0) * RM + row;
-    if ((G & 3) == 0) {
-        constexpr int B = kTransposeGroups / 4;
-        float4 v[B];
-#pragma unroll
-        for (int j = 0; j < B; ++j) v[j] = (4 * j < n) ? *(const float4*)(sp + 4 * j) : make_float4(0, 0, 0, 0);
-        if (valid) {
-#pragma unroll
-            for (int j = 0; j < B; ++j) {
-                if (4 * j >= n) break;
-                dp[(int64_t)(4 * j + 0) * RM] = v[j].x;
-                dp[(int64_t)(4 * j + 1) * RM] = v[j].y;
-                dp[(int64_t)(4 * j + 2) * RM] = v[j].z;
-                dp[(int64_t)(4 * j + 3) * RM] = v[j].w;
-            }
-        }
-    } else if (valid) {
-        for (int g = 0; g < n; ++g) dp[(int64_t)g * RM] = sp[g];
     }
 }
 
@@ -798,14 +812,22 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
                                                              const void* __restrict__ zero_row,
                                                              const float* __restrict__ factor, int R, int E, int K,
                                                              int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
-                                                             int total_tasks) {
+                                                             int group_blocks) {
     constexpr int kSlab = FP8 ? 1024 : 512;
     constexpr int kLaneElems = kSlab / 64;
     const int lane = wave_lane();
-    const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
-    if (task >= total_tasks) return;
-    const int n = task / slabs, s = task - n * slabs;
-    const int r = n / Tgrid, t = n - r * Tgrid;
+    // Blocks go round-robin over the 8 XCDs, each with an L2 of its own.  The rows that one source rank
+    // sent to an expert are neighbours in the expert's block, so their scales of one group share 64-byte
+    // sectors: all the waves of a (rank, slab) pair - the ones that read those sectors - are therefore
+    // given to one XCD, next to each other in launch order (group_blocks consecutive blocks of that XCD).
+    const int wpb = blockDim.x >> 6;
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int gl = seq / group_blocks, tb = seq - gl * group_blocks;
+    const int gid = gl * 8 + xcd;
+    if (gid >= R * slabs) return;
+    const int r = gid / slabs, s = gid - r * slabs;
+    const int t = __builtin_amdgcn_readfirstlane(tb * wpb + (threadIdx.x >> 6));
+    if (t >= Tgrid) return;
     const int T = cs.tokens >= 0 ? cs.tokens : (int)tbl[CF_NUM_TOKENS * R + r];
     if (t >= T) return;
     char* orow = (char*)rank_ptr(tbl, cs.out, CF_OUT, R, r) + (int64_t)t * H * 2;
@@ -913,7 +935,7 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
 #pragma unroll
     for (int j = 0; j < kLaneElems / 2; ++j) o[j] = pack_bf16_rne(acc[2 * j], acc[2 * j + 1]);
     store16<true>(orow + (int64_t)elem * 2, make_uint4(o[0], o[1], o[2], o[3]));
-    if (FP8) store16<true>(orow + (int64_t)elem * 2 + 16, make_uint4(o[4], o[5], o[6], o[7]));
+    if constexpr (FP8) store16<true>(orow + (int64_t)elem * 2 + 16, make_uint4(o[4], o[5], o[6], o[7]));
 }
 
 // Work list of the cast-back kernel: which (expert, row chunk) each chunk
@@ -1086,6 +1108,48 @@ __global__ __launch_bounds__(256) void copy_kernel(uint4* __restrict__ dst, cons
     for (; i < n; i += stride) dst[i] = src[i];
 }
 
+// Synthetic streams with the read : write mixes of the data kernels, one 16-byte unit per thread and
+// nothing else: what this GPU's memory system gives each mix when no routing, arithmetic or row
+// structure is in the way (the ceilings the data kernels are compared with).
+//   0 copy      read n, write n units                         (1 : 1)
+//   1 read      read n units, write nothing
+//   2 write     write n units
+//   3 widen     read n half units (8 bytes), write n units    (1 : 2, the cast-back kernel's mix)
+//   4 gather8   read 8 streams of n units, write n            (8 : 1, the reduce kernel's mix)
+//   5 scatter8  read 2n units, write 8 streams of n           (1 : 4, the fp8 pack kernel's mix)
+template <int KIND>
+__global__ __launch_bounds__(256) void stream_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                                      size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    if (KIND == 0) {
+        dst[i] = src[i];
+    } else if (KIND == 1) {
+        const uint4 v = load16<true>(src + i);
+        if (v.x == 0x12345678u && v.y == 0x9abcdef0u && v.z == 1u && v.w == 2u) dst[0] = v;   // never, in practice
+    } else if (KIND == 2) {
+        dst[i] = make_uint4((uint32_t)i, 1u, 2u, 3u);
+    } else if (KIND == 3) {
+        const uint2 v = ((const uint2*)src)[i];
+        dst[i] = make_uint4(v.x, v.y, v.x ^ v.y, v.x + v.y);
+    } else if (KIND == 4) {
+        uint4 v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = load16<true>(src + (size_t)k * n + i);
+        uint4 a = v[0];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) {
+            a.x ^= v[k].x; a.y ^= v[k].y; a.z ^= v[k].z; a.w ^= v[k].w;
+        }
+        store16<true>(dst + i, a);
+    } else {
+        const uint4 a = load16<true>(src + 2 * i), b = load16<true>(src + 2 * i + 1);
+        const uint4 o = make_uint4(a.x ^ b.x, a.y ^ b.y, a.z ^ b.z, a.w ^ b.w);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) dst[(size_t)k * n + i] = o;
+    }
+}
+
 __global__ __launch_bounds__(256) void fill_kernel(uint32_t* __restrict__ dst, uint32_t value, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -1178,6 +1242,15 @@ hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const D
 
 static int clamp_waves(int w) { return w < 1 ? 1 : (w > kMaxPackWaves ? kMaxPackWaves : w); }
 
+static long long transpose_items(const Dims& d, int* parts_out) {
+    const int G = d.H / 128;
+    const int parts = (G + kTransposeGroups - 1) / kTransposeGroups;
+    // every selection is at most one row, and each expert has at most one partly filled chunk
+    const long long chunks = ((long long)d.R * d.Tgrid * d.K + 63) / 64 + d.E;
+    *parts_out = parts;
+    return chunks * parts;
+}
+
 template <typename Kern>
 static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src,
                                 float* stage, const Dims& d, const Tuning& t, hipStream_t stream) {
@@ -1202,27 +1275,22 @@ hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const Di
     if (use_fp8 && scale_stage == nullptr) return hipErrorInvalidValue;
     hipError_t err = hipSuccess;
     if (run_pack) {
+#define MCEP_PF(A, B) launch_pack_t(pack_fp8_kernel<A, B>, d_tbl, sc, src, scale_stage, d, t, stream)
         if (!use_fp8)
             err = ntl ? launch_pack_t(pack_bf16_kernel<true>, d_tbl, sc, src, scale_stage, d, t, stream)
                       : launch_pack_t(pack_bf16_kernel<false>, d_tbl, sc, src, scale_stage, d, t, stream);
-        else if (t.fp8_arith == 1)
-            err = ntl ? launch_pack_t(pack_fp8_kernel<true, true>, d_tbl, sc, src, scale_stage, d, t, stream)
-                      : launch_pack_t(pack_fp8_kernel<false, true>, d_tbl, sc, src, scale_stage, d, t, stream);
         else
-            err = ntl ? launch_pack_t(pack_fp8_kernel<true, false>, d_tbl, sc, src, scale_stage, d, t, stream)
-                      : launch_pack_t(pack_fp8_kernel<false, false>, d_tbl, sc, src, scale_stage, d, t, stream);
+            err = ntl ? (t.fp8_arith == 1 ? MCEP_PF(true, true) : MCEP_PF(true, false))
+                      : (t.fp8_arith == 1 ? MCEP_PF(false, true) : MCEP_PF(false, false));
+#undef MCEP_PF
     }
     if (err != hipSuccess || !use_fp8 || !run_finish) return err;
-    float* stage = scale_stage;
-    const int G = d.H / 128;
-    const int parts = (G + kTransposeGroups - 1) / kTransposeGroups;
-    // every selection is at most one row, and each expert has at most one partly filled chunk
-    const long long chunks = ((long long)d.R * d.Tgrid * d.K + 63) / 64 + d.E;
-    const long long total = chunks * parts;
-    if (total > 0x7fffffffll) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(scale_transpose_kernel, dim3((unsigned)((total + kTransposeWaves - 1) / kTransposeWaves)),
-                       dim3(kTransposeWaves * 64), 0, stream, d_tbl, stage, sc, d.R, d.E, G, d.max_tokens, parts,
-                       (int)total);
+    int parts = 1;
+    const long long items = transpose_items(d, &parts);
+    if (items > 0x7fffffffll) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(scale_transpose_kernel, dim3((unsigned)((items + kTransposeWaves - 1) / kTransposeWaves)),
+                       dim3(kTransposeWaves * 64), 0, stream, d_tbl, scale_stage, sc, d.R, d.E, d.H / 128, d.max_tokens,
+                       parts, (int)items);
     return hipGetLastError();
 }
 
@@ -1302,14 +1370,16 @@ static hipError_t launch_reduce_packed_t(const ReduceLaunch& rl, const float* d_
                                          hipStream_t stream) {
     const int slab = FP8 ? 1024 : 512;
     const int slabs = (d.H + slab - 1) / slab;
-    const long long total = (long long)d.R * d.Tgrid * slabs;
-    if (total <= 0) return hipSuccess;
-    if (total > 0x7fffffffll) return hipErrorInvalidValue;
+    if (d.Tgrid <= 0) return hipSuccess;
     const int wpb = clamp_waves(t.combine_waves);
-    const int blocks = (int)((total + wpb - 1) / wpb);
-    hipLaunchKernelGGL((reduce_packed_kernel<KMAX, FP8, FACTOR, DIRECT>), dim3(blocks), dim3(wpb * 64), 0, stream,
-                       rl.d_tbl, rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d_factor, d.R, d.E, d.K,
-                       d.max_tokens, d.H, d.plan, slabs, d.Tgrid, (int)total);
+    // (rank, slab) groups, eight at a time (one per XCD), each a run of group_blocks blocks
+    const int group_blocks = (d.Tgrid + wpb - 1) / wpb;
+    const long long rounds = ((long long)d.R * slabs + 7) / 8;
+    const long long blocks = rounds * 8 * group_blocks;
+    if (blocks > 0x7fffffffll) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((reduce_packed_kernel<KMAX, FP8, FACTOR, DIRECT>), dim3((unsigned)blocks), dim3(wpb * 64), 0,
+                       stream, rl.d_tbl, rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d_factor, d.R, d.E, d.K,
+                       d.max_tokens, d.H, d.plan, slabs, d.Tgrid, group_blocks);
     return hipGetLastError();
 }
 
@@ -1368,6 +1438,25 @@ hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t str
     size_t blocks = (n + 255) / 256;
     if (blocks > 256 * 64) blocks = 256 * 64;
     hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_stream(int kind, void* dst, const void* src, size_t unit_bytes, hipStream_t stream) {
+    const size_t n = unit_bytes / 16;
+    if (n == 0) return hipSuccess;
+    const size_t blocks = (n + 255) / 256;
+    if (blocks > 0x7fffffffull || kind < 0 || kind > 5) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)blocks), block(256);
+    uint4* d = (uint4*)dst;
+    const uint4* s = (const uint4*)src;
+    switch (kind) {
+        case 0: hipLaunchKernelGGL(stream_kernel<0>, grid, block, 0, stream, d, s, n); break;
+        case 1: hipLaunchKernelGGL(stream_kernel<1>, grid, block, 0, stream, d, s, n); break;
+        case 2: hipLaunchKernelGGL(stream_kernel<2>, grid, block, 0, stream, d, s, n); break;
+        case 3: hipLaunchKernelGGL(stream_kernel<3>, grid, block, 0, stream, d, s, n); break;
+        case 4: hipLaunchKernelGGL(stream_kernel<4>, grid, block, 0, stream, d, s, n); break;
+        default: hipLaunchKernelGGL(stream_kernel<5>, grid, block, 0, stream, d, s, n); break;
+    }
     return hipGetLastError();
 }
 
