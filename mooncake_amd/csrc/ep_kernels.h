@@ -82,6 +82,8 @@ struct RoutingScratch {
     int32_t* ucount_t;   // [E, kMaxSummedUnits]  the same, expert-major (summed plan only)
     int32_t* ubegin;     // [U, E]  exclusive prefix of ucount over units
     int32_t* selpos;     // [R * max_tokens * K]  position inside (unit, expert); -1: no valid expert
+    int32_t* selrow;     // [R * max_tokens * K]  expert * R*max + packed row of the selection, -1: none; left by the
+                         //                       pack kernel for a combine of the same handle
     int32_t* counts;     // [E]     rows per expert (0 for experts of ranks that take no part)
     int32_t* row_src;    // [E, R * max_tokens]  packed row -> source token slot (rank * max_tokens + token)
 };
@@ -110,6 +112,8 @@ struct DispatchSource {
 
 struct CombineSource {
     RankPtr topk_idx, topk_weights, out;
+    RankPtr x;              // the rows combine reads (expert outputs, or the packed payload)
+    RankPtr scales;         // packed combine of an fp8 payload
     int tokens = -1;
 };
 

@@ -469,8 +469,11 @@ __device__ __forceinline__ PackDest pack_destination(const uint64_t* __restrict_
     const int ub = up.summed ? summed_begin(sc, k, up, r, t, K, j, stride) : sc.ubegin[(int64_t)k.unit * E + k.e];
     const SelRow s = selection_row(k, ub, R, max_tokens);
     PackDest d = {0};
+    const int64_t RM = (int64_t)R * max_tokens;
+    // where the selection went, for a combine of this dispatch's handle: expert * R*max + row, or -1
+    if (slab == 0 && j == 0 && slot < K)
+        sc.selrow[((int64_t)r * max_tokens + t) * K + slot] = (s.ok && base != 0) ? (int)((int64_t)k.e * RM + s.slot) : -1;
     if (s.ok && base != 0) {
-        const int64_t RM = (int64_t)R * max_tokens;
         d.row = base + (uint64_t)s.grow * (uint64_t)H * (FP8 ? 1 : 2);
         if (slab == 0 && j == 0) {
             ((int32_t*)info)[s.grow] = t;
@@ -676,6 +679,38 @@ __global__ __launch_bounds__(256) void resolve_kernel(const uint64_t* __restrict
     }
 }
 
+// Where combine finds the row of selection `lane` of token (r, t) when the handle is the last
+// dispatch's: the pack kernel left expert * R*max + row in selrow (-1: the selection went nowhere).
+// One load away from the payload when the ranks' row tensors are evenly spaced (the address then comes
+// from kernel arguments), two otherwise (rank table).  `live` is loaded but not waited for: whether
+// the owner is active only decides the weight, so the caller issues its payload loads first.
+struct DirectRow {
+    uint64_t base;      // the owner's row tensor, 0: none
+    int64_t grow;       // row inside the owner's [L, R*max] layout
+    int e, q, le, slot;
+    int live;           // the token owner's active_ranks entry for the expert's rank
+    bool has;
+};
+
+__device__ __forceinline__ DirectRow direct_row(const uint64_t* __restrict__ tbl, const RoutingScratch& sc,
+                                                const RankPtr& x, int R, int E, int K, int max_tokens, int r, int t,
+                                                int lane) {
+    const int RM = R * max_tokens;
+    const int L = E / R;
+    const int32_t* active = (const int32_t*)tbl[CF_ACTIVE * R + r];
+    const int sr = sc.selrow[((int64_t)r * max_tokens + t) * K + (lane < K ? lane : 0)];
+    DirectRow d;
+    d.has = lane < K && sr >= 0;
+    d.e = d.has ? sr / RM : 0;
+    d.slot = d.has ? sr - d.e * RM : 0;
+    d.q = d.e / L;
+    d.le = d.e - d.q * L;
+    d.base = rank_ptr(tbl, x, CF_X, R, d.q);
+    d.live = active[d.q];
+    d.grow = (int64_t)d.le * RM + d.slot;
+    return d;
+}
+
 // One wave per (token, slab of CH * 512 elements).  Lanes 0..K-1 find the K
 // source rows (a masked, inactive or unknown selection reads a zero row with
 // weight 0, which leaves the fp32 accumulator unchanged), then every lane
@@ -700,23 +735,18 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
 
     uint64_t src = (uint64_t)zero_row;
     float w = 0.0f;
+    int live = 1;
     if (DIRECT) {
         // the caller's top-k rows exist only for t < T
         if (t >= T) return;
-        const int64_t* idx_row = (const int64_t*)rank_ptr(tbl, cs.topk_idx, CF_TOPK_IDX, R, r) + (int64_t)t * K;
         const float* w_row = (const float*)rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (int64_t)t * K;
         const float wl = w_row[lane < K ? lane : 0];
-        const int32_t* active = (const int32_t*)tbl[CF_ACTIVE * R + r];
-        const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, up, r, t, lane);
-        // the dependent gathers, side by side
-        const int ub = sc.ubegin[(int64_t)k.unit * E + k.e];
-        const uint64_t base = tbl[CF_X * R + k.q];
-        const int live = active[k.q];                          // skip experts on inactive ranks
-        const SelRow sr = selection_row(k, ub, R, max_tokens);
-        if (sr.ok && base != 0 && live != 0) {
-            src = base + (uint64_t)sr.grow * (uint64_t)H * 2;
+        const DirectRow d = direct_row(tbl, sc, cs.x, R, E, K, max_tokens, r, t, lane);
+        if (d.has && d.base != 0) {
+            src = d.base + (uint64_t)d.grow * (uint64_t)H * 2;
             w = wl;
         }
+        live = d.live;         // not looked at before the payload loads are on their way
     } else {
         // A token slot beyond the rank's count has only stale routes (zero
         // rows); it is computed like any other and dropped at the store, so
@@ -743,9 +773,20 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
         const uint64_t p = read_lane_u64(src, k);
-        wk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k));
 #pragma unroll
         for (int c = 0; c < CH; ++c) v[k][c] = load16<NTL>((const void*)(p + off[c]));
+    }
+    // An expert on a rank the token's owner sees as inactive is skipped (mooncake_ep_kernel.cu:729-732):
+    // its row was fetched before that was known, so the row is dropped here (it may hold anything) and
+    // the weight is zero, as for a selection that went nowhere.
+    if (DIRECT && live == 0) w = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        wk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k));
+        if (DIRECT && __builtin_amdgcn_readlane(live, k) == 0) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) v[k][c] = make_uint4(0, 0, 0, 0);
+        }
     }
 
     if (t >= T) return;
@@ -838,22 +879,19 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
     uint64_t src = (uint64_t)zero_row, ssrc = (uint64_t)zero_row;
     float w = 0.0f, f = 1.0f;
     int sstride = 0;                     // bytes between a row's consecutive scale groups (0: the zero row)
+    int live = 1;                        // DIRECT: loaded here, looked at after the payload loads are issued
     {
         int e = 0, slot = 0;
         bool ok = false;
         float wl = 0.0f;
         if (DIRECT) {
-            const int64_t* idx_row = (const int64_t*)rank_ptr(tbl, cs.topk_idx, CF_TOPK_IDX, R, r) + (int64_t)t * K;
             const float* w_row = (const float*)rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (int64_t)t * K;
             wl = w_row[lane < K ? lane : 0];
-            const int32_t* active = (const int32_t*)tbl[CF_ACTIVE * R + r];
-            const SelKey k = selection_key(idx_row, sc, R, E, K, max_tokens, up, r, t, lane);
-            const int ub = sc.ubegin[(int64_t)k.unit * E + k.e];
-            const int live = active[k.q];                      // skip experts on inactive ranks
-            const SelRow sr = selection_row(k, ub, R, max_tokens);
-            ok = sr.ok && live != 0;
-            e = k.e;
-            slot = sr.slot;
+            const DirectRow d = direct_row(tbl, sc, cs.x, R, E, K, max_tokens, r, t, lane);
+            ok = d.has;
+            e = d.e;
+            slot = d.slot;
+            live = d.live;
         } else {
             uint4 rt = make_uint4(0, 0, 0, 0);
             if (lane < K) rt = *(const uint4*)(routes + ((int64_t)r * max_tokens + t) * K + lane);
@@ -863,8 +901,8 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
             wl = __uint_as_float(rt.z);
         }
         const int q = e / L, le = e - q * L;
-        const uint64_t base = tbl[CF_X * R + q];
-        const uint64_t sbase = FP8 ? tbl[CF_SCALES * R + q] : 0;
+        const uint64_t base = rank_ptr(tbl, cs.x, CF_X, R, q);
+        const uint64_t sbase = FP8 ? rank_ptr(tbl, cs.scales, CF_SCALES, R, q) : 0;
         const float fe = FACTOR ? factor[e] : 1.0f;
         if (ok && base != 0 && (!FP8 || sbase != 0)) {
             const int64_t grow = (int64_t)le * RM + slot;
@@ -888,7 +926,6 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
         const uint64_t p = read_lane_u64(src, k);
-        wk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k));
         fk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), k));
         v[k] = load16<true>((const void*)(p + poff));
         if (FP8) {
@@ -900,6 +937,16 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
         }
     }
 
+    // a row of a rank the token's owner sees as inactive was fetched before that was known: drop it
+    if (DIRECT && live == 0) w = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        wk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k));
+        if (DIRECT && __builtin_amdgcn_readlane(live, k) == 0) {
+            v[k] = make_uint4(0, 0, 0, 0);
+            sv[k] = 0.0f;
+        }
+    }
     float acc[kLaneElems];
 #pragma unroll
     for (int j = 0; j < kLaneElems; ++j) acc[j] = 0.0f;

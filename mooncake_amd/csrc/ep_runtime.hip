@@ -159,6 +159,8 @@ struct mc_ep_world {
     size_t ucount_t_cap = 0;
     int32_t* d_selpos = nullptr;
     size_t selpos_cap = 0;
+    int32_t* d_selrow = nullptr;
+    size_t selrow_cap = 0;
     int32_t* d_row_src = nullptr;
     size_t row_src_cap = 0;
     int32_t* d_counts = nullptr;
@@ -202,7 +204,7 @@ struct mc_ep_world {
         const bool switched = hipGetDevice(&prev) == hipSuccess && prev != device && hipSetDevice(device) == hipSuccess;
         (void)hipDeviceSynchronize();
         void* owned[] = {d_tbl[0], d_tbl[1], d_tbl[2], d_captured_tbl[0], d_captured_tbl[1], d_captured_tbl[2],
-                         d_ucount, d_ucount_t, d_ubegin, d_selpos, d_row_src, d_counts, d_chunk_map, d_routes,
+                         d_ucount, d_ucount_t, d_ubegin, d_selpos, d_selrow, d_row_src, d_counts, d_chunk_map, d_routes,
                          d_scale_stage, d_zero_row};
         for (void* p : owned)
             if (p) (void)hipFree(p);
@@ -391,7 +393,7 @@ int uniform_tokens(const int32_t* n, int R, bool enabled) {
 }
 
 RoutingScratch routing_scratch(const mc_ep_world* w) {
-    return RoutingScratch{w->d_ucount, w->d_ucount_t, w->d_ubegin, w->d_selpos, w->d_counts, w->d_row_src};
+    return RoutingScratch{w->d_ucount, w->d_ucount_t, w->d_ubegin, w->d_selpos, w->d_selrow, w->d_counts, w->d_row_src};
 }
 
 // Enqueues what is left of a round that was launched in two parts (see Round::finish).
@@ -492,6 +494,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         sc.ucount_t = (int32_t*)carve((size_t)num_experts * kMaxSummedUnits * 4);
         sc.ubegin = (int32_t*)carve(UE * 4);
         sc.selpos = (int32_t*)carve((size_t)R * max_tokens * num_topk * 4);
+        sc.selrow = (int32_t*)carve((size_t)R * max_tokens * num_topk * 4);
         sc.counts = (int32_t*)carve((size_t)num_experts * 4);
         sc.row_src = (int32_t*)carve((size_t)num_experts * R * max_tokens * 4);
         stage = (float*)carve(stage_floats * 4);
@@ -513,6 +516,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         if (int rc = ensure_scratch(w, &w->d_ubegin, &w->ubegin_cap, UE)) return rc;
         if (int rc = ensure_scratch(w, &w->d_ucount_t, &w->ucount_t_cap, (size_t)num_experts * kMaxSummedUnits)) return rc;
         if (int rc = ensure_scratch(w, &w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
+        if (int rc = ensure_scratch(w, &w->d_selrow, &w->selrow_cap, (size_t)R * max_tokens * num_topk)) return rc;
         if (int rc = ensure_scratch(w, &w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
         if (int rc = ensure_scratch(w, &w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
         if (stage_floats > 0 && (phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
@@ -611,7 +615,8 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     // the combine of its handle (mooncake_ep_kernel.cu:734 finds a token's rows
     // by its dispatch-time expert indices).
     const auto& ld = w->last;
-    bool direct = w->tuning.combine_direct != 0 && ld.valid && ld.data_done && ld.hidden == hidden && ld.num_topk == num_topk &&
+    bool direct = w->tuning.combine_direct != 0 && ld.valid && ld.data_done && ld.hidden == hidden &&
+                  (long long)num_experts * R * max_tokens < 0x7fffffffll && ld.num_topk == num_topk &&
                   ld.max_tokens == max_tokens && ld.num_experts == num_experts;
     // "Last" is about the order on the device.  Graph replays run dispatches the host never sees, so: a
     // recorded combine trusts only a dispatch recorded in the same capture, and once a dispatch of this
@@ -628,6 +633,8 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     src.topk_idx = uniform_ptr(topk_idx, R, uni);
     src.topk_weights = uniform_ptr(topk_weights, R, uni);
     src.out = uniform_ptr(out, R, uni);
+    src.x = uniform_ptr(x, R, uni);
+    if (ps.scales != nullptr) src.scales = uniform_ptr(ps.scales, R, uni);
     src.tokens = uniform_tokens(num_tokens, R, uni);
     // sized on every path, so that an eager call prepares the world for any recorded one of the same shape
     if (int rc = ensure_routes(w, (size_t)R * max_tokens * num_topk)) return rc;
