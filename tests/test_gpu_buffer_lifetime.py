@@ -140,6 +140,64 @@ def test_two_streams_alternate_on_one_world_without_waits(gpu_device, oracle, us
         assert torch.equal(h.combined.cpu().view(torch.int16), want.view(torch.int16)), f"data set {i}"
 
 
+@pytest.mark.parametrize("mode", ["default", "async", "hook"])
+def test_every_rank_on_a_stream_of_its_own(gpu_device, oracle, mode):
+    """Callers on different streams: the round runs on the world's communication stream, after what each
+    rank's stream holds, and each rank's later work (default: at once; async / hook: after the wait) sees it."""
+    R, T, H, E, K = 4, 96, 2048, 32, 4
+    announce(f"one stream per rank, {mode}")
+    world, bufs = make_world(R, T, H, E)
+    streams = [torch.cuda.Stream() for _ in range(R)]
+    ins = [rank_inputs(700 + r, T, H, E, K) for r in range(R)]
+    host = [tuple(t.pin_memory() for t in i) for i in ins]
+    dev, outs, sums = [None] * R, [None] * R, [None] * R
+    kw = dict(async_finish=mode == "async", return_recv_hook=mode == "hook")
+    for r in range(R):
+        with torch.cuda.stream(streams[r]):
+            # the inputs arrive on the rank's own stream right before the call: the round must wait for that
+            dev[r] = tuple(t.to(gpu_device, non_blocking=True) for t in host[r])
+            outs[r] = bufs[r].dispatch(dev[r][0], dev[r][1], None, T, E, -1, use_fp8=True, **kw)
+    for r in range(R):
+        with torch.cuda.stream(streams[r]):
+            if mode == "async":
+                outs[r][3].current_stream_wait()
+            if mode == "hook":
+                outs[r][4]()
+            # a consumer on the rank's stream, with nothing but the library between it and the round
+            sums[r] = outs[r][1].sum()
+    torch.cuda.synchronize()
+    ref, *_ = oracle_world(oracle, ins, T, E, True)
+    for r in range(R):
+        assert int(sums[r]) == int(ref["recv_count"][r].sum())
+        check_rank_dispatch(ref, r, outs[r][0], outs[r][1], outs[r][2], True)
+    # combine the same way
+    factor = torch.arange(E, dtype=torch.float32) * 0.1 + 1.0
+    rows = oracle.cast_back(ref["recv_x"], ref["scales"], ref["recv_count"], factor)
+    nt = [T] * R
+    xs = torch.stack([i[0] for i in ins]); idxs = torch.stack([i[1] for i in ins]); ws = torch.stack([i[2] for i in ins])
+    want = oracle.combine(rows, idxs, ws, ref["src_info"], ref["layout_range"], nt, T, E)
+    L = E // R
+    res = [None] * R
+    for r in range(R):
+        with torch.cuda.stream(streams[r]):
+            (px, ps), cnt, handle, _, _ = outs[r]
+            f = factor[r * L:(r + 1) * L].to(gpu_device, non_blocking=True).view(L, 1, 1)
+            once = (px.float().view(L, R * T, H // 128, 128) * ps.unsqueeze(-1)).view(L, R * T, H).to(torch.bfloat16)
+            eo = (once.float() * f).to(torch.bfloat16)
+            res[r] = bufs[r].combine(eo, dev[r][1], dev[r][2], None, -1, handle, **kw)
+    copies = [None] * R
+    for r in range(R):
+        with torch.cuda.stream(streams[r]):
+            if mode == "async":
+                res[r][1].current_stream_wait()
+            if mode == "hook":
+                res[r][2]()
+            copies[r] = res[r][0].clone()
+    torch.cuda.synchronize()
+    for r in range(R):
+        assert torch.equal(copies[r].cpu().view(torch.int16), want[r].view(torch.int16)), f"rank {r}"
+
+
 def test_rank_dies_between_dispatch_and_combine(gpu_device, oracle):
     # test_ep_grid.py:250-369 at its shape family: 2 ranks, bf16, async_finish, fail_rank 1
     R, T, H, E, K = 2, 128, 2048, 32, 4
