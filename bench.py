@@ -63,6 +63,10 @@ def parse_args():
     ap.add_argument("--stream-ceilings", action="store_true",
                     help="instead of the workload, time synthetic streams with the data kernels' read : write mixes "
                          "and byte counts (what the memory system gives each mix), and print them as JSON")
+    ap.add_argument("--kernel-pass", type=int, default=0, metavar="N",
+                    help="instead of timing, run every kernel of the workload (dispatch, cast_back, combine, packed "
+                         "combine) and the synthetic streams sized like them N times and exit: the program to put "
+                         "under `rocprofv3 --pmc` when comparing hardware counters of the two")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (the known-size "
                          "kernel that profiler FETCH_SIZE / WRITE_SIZE readings are scaled against)")
@@ -353,6 +357,28 @@ def main():
 
     if args.stream_ceilings:
         print(json.dumps({"workload": cfg.name, "stream_ceilings": stream_ceilings(cfg, S, args.kernel_iters)}))
+        return
+
+    if args.kernel_pass > 0:
+        h = WorldHarness(cfg, device="cuda:0")
+        h.load(data)
+        h.alloc_dispatch_outputs()
+        h.alloc_combine_io()
+        lib, stream = _lib.lib(), int(torch.cuda.current_stream().cuda_stream)
+        H, N = cfg.hidden, cfg.total_tokens
+        big = S * H * 2
+        src = torch.empty(big, dtype=torch.uint8, device="cuda:0").fill_(3)
+        dst = torch.empty(big, dtype=torch.uint8, device="cuda:0")
+        for _ in range(args.kernel_pass):
+            h.dispatch()
+            h.cast_back()
+            h.combine()
+            h.combine_packed()
+            # gather 8:1 sized like the reduce kernel, scatter 1:4 like the fp8 pack kernel, widen 1:2 like cast_back
+            for kind, unit_bytes in ((4, N * H * 2), (5, S * H // 8), (3, S * H * 2)):
+                _lib.check(lib.mc_ep_debug_stream(kind, dst.data_ptr(), src.data_ptr(), unit_bytes // 4096 * 4096, stream))
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": cfg.name, "kernel_pass": args.kernel_pass}))
         return
 
     h = WorldHarness(cfg, device="cuda:0")
