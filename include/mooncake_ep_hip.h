@@ -14,7 +14,14 @@
  * where this ABI returns MC_EP_ERR_ASSERT with the same condition text.
  *
  * Not thread-safe per object, like the reference
- * (mooncake_ep_buffer.cpp:215-218): drive one world from one thread.
+ * (mooncake_ep_buffer.cpp:215-218): drive one world from one thread.  The
+ * calls of one world share its scratch (rank tables, routing state, staged
+ * scales), so the library serialises them across streams: a call on another
+ * stream than the world's previous call first waits for what that stream
+ * holds.  A stream that has carried a world's calls must therefore stay valid
+ * while later calls of the world may follow on other streams.  Scratch grows
+ * by replacement; outgrown allocations are kept until the world is destroyed,
+ * because queued kernels and instantiated graphs hold their addresses.
  */
 #ifndef MOONCAKE_EP_HIP_H
 #define MOONCAKE_EP_HIP_H
@@ -75,10 +82,16 @@ int mc_ep_world_num_ranks(const mc_ep_world_t* world);
  * rank has opened yet. */
 int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
 
-/* Tuning knobs for measurement sweeps ("pack_variant", "pack_waves",
- * "combine_chunks", "combine_waves", "combine_nt", "combine_direct", "uniform",
- * "pack_nt",
- * "scale_mode", "routing_sum"). */
+/* Options ("pack_waves", "pack_nt", "uniform", "routing_sum", "combine_direct",
+ * "combine_chunks", "combine_waves", "combine_nt": tuning knobs for measurement
+ * sweeps; "fp8_arith": 0 (default) the fp8 scale arithmetic of the reference's
+ * PyTorch statement as CPU PyTorch runs it - 448.0 / amax as reciprocal times
+ * 448, amax / 448.0 a true division (mooncake_ep_buffer.py:699-702) - or 1 the
+ * reference kernel's own, 448 / amax as one IEEE division and amax * (1 / 448)
+ * (mooncake_ep_kernel.cu:184, :252), which differ in the last bit of a scale
+ * for about a quarter of all groups; "comm_stream": 1 runs every per-rank
+ * collective on the world's communication stream as the reference does, 0
+ * (default) on the callers' stream when they all share one). */
 int mc_ep_world_set_option(mc_ep_world_t* world, const char* name, int value);
 int mc_ep_world_get_option(const mc_ep_world_t* world, const char* name, int* value);
 
@@ -109,9 +122,9 @@ int mc_ep_world_dispatch(mc_ep_world_t* world, const uint64_t* x_ptrs, const uin
  * 16 MiB array in static device memory that each GPU the library runs on holds
  * until the process ends.  A shape that needs more (about
  * num_experts * num_ranks * max_tokens * 4 bytes, plus
- * num_ranks * max_tokens * (num_topk * 4 + hidden / 32) bytes) is rejected with
+ * num_ranks * max_tokens * (num_topk * 8 + hidden / 32) bytes) is rejected with
  * MC_EP_ERR_ASSERT and a message that says so; the DeepSeek-V3 decode world
- * (32 x 128 tokens, 256 experts, hidden 7168) needs 5.3 MB.  Same arguments,
+ * (32 x 128 tokens, 256 experts, hidden 7168) needs 5.5 MB.  Same arguments,
  * outputs and errors as mc_ep_world_dispatch otherwise.  Every call on a GPU,
  * from any world, shares that GPU's array and overwrites the last call's
  * contents: calls that overlap on one GPU (different streams without an order

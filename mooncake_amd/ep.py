@@ -21,6 +21,11 @@ import os
 from ctypes import c_void_p
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
+# PyTorch first, as in the reference's ep.py (mooncake-wheel/mooncake/ep.py:4): a ROCm build of PyTorch ships
+# its own HIP runtime, and the library must bind to that one - the runtime that owns the tensors it is handed -
+# rather than bring a second one into the process by being loaded before it.
+import torch  # noqa: F401
+
 from . import _lib
 
 MAX_QP_COUNT = 256   # mooncake_ep_configs.cuh:5
