@@ -218,7 +218,7 @@ def test_rank_dies_between_dispatch_and_combine(gpu_device, oracle):
         factor = (torch.arange(r * L, (r + 1) * L, device=gpu_device).float() * 0.1 + 1.0).view(L, 1, 1)
         return (recv_x.float() * factor).to(torch.bfloat16)
 
-    # round 1: every rank alive, on the buffers round 2 will reuse
+    # first cycle: every rank alive, on the buffers the second cycle reuses
     nts = [T, int(T * (1.0 - 0.05 * (1 / R)))]
     ins, act, outs = dispatch_all(2026, nts)
     combined = []
@@ -234,7 +234,7 @@ def test_rank_dies_between_dispatch_and_combine(gpu_device, oracle):
         want = (x.float() * ((idx.float() * 0.1 + 1.0) * w).sum(dim=1, keepdim=True)).to(torch.bfloat16)
         torch.testing.assert_close(combined[r][0], want, rtol=5e-2, atol=1e-3)
 
-    # round 2: both dispatch, rank 1 goes away before combine
+    # second cycle: both ranks dispatch, rank 1 goes away before combine
     ins, act, outs = dispatch_all(200, nts)
     torch.cuda.synchronize()
     world.set_rank_silent(fail)
