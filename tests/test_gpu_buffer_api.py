@@ -23,10 +23,10 @@ from tests.gpu_util import announce
 pytestmark = pytest.mark.gpu
 
 
-def make_world(num_ranks, max_tokens, hidden, num_experts):
+def make_world(num_ranks, max_tokens, hidden, num_experts, disable_p2p=False):
     world, groups = LogicalGroup.make_world(num_ranks)
     nbytes = Buffer.get_ep_buffer_size_hint(max_tokens, hidden, num_ranks, num_experts)
-    return world, [Buffer(g, nbytes) for g in groups]
+    return world, [Buffer(g, nbytes, disable_p2p=disable_p2p) for g in groups]
 
 
 def grid_inputs(rank, num_ranks, max_tokens, hidden, num_experts, top_k, device):
@@ -51,13 +51,18 @@ MODES = [(False, False), (True, False), (False, True)]      # (async_finish, ret
 
 @pytest.mark.parametrize("use_fp8", [False, True], ids=["bf16", "fp8"])
 @pytest.mark.parametrize("async_finish,return_recv_hook", MODES, ids=["default", "async", "hook"])
-@pytest.mark.parametrize("fail_rank", [-1, 2], ids=["all_alive", "rank2_dead"])
+@pytest.mark.parametrize("fail_rank", [-1, 1], ids=["all_alive", "rank1_dead"])
+@pytest.mark.parametrize("disable_p2p", [False, True], ids=["p2p", "no_p2p"])
 @pytest.mark.parametrize("comm_stream", [0, 1], ids=["callers_stream", "comm_stream"])
-def test_grid_closed_form(gpu_device, oracle, use_fp8, async_finish, return_recv_hook, fail_rank, comm_stream):
-    num_ranks, max_tokens, hidden, num_experts, top_k = 4, 256, 2048, 288, 8
+def test_grid_closed_form(gpu_device, oracle, use_fp8, async_finish, return_recv_hook, fail_rank, disable_p2p,
+                          comm_stream):
+    # the reference's grid (test_ep_grid.py:469-483): fp8 x async x hook x fail_rank {-1, 1} x disable_p2p at its one
+    # shape, on 8 ranks (its world is one rank per GPU of a node); use_fallback has no counterpart here
+    num_ranks, max_tokens, hidden, num_experts, top_k = 8, 256, 2048, 288, 8
     announce(f"grid fp8={use_fp8} async={async_finish} hook={return_recv_hook} fail_rank={fail_rank} "
-             f"comm_stream={comm_stream}")
-    world, bufs = make_world(num_ranks, max_tokens, hidden, num_experts)
+             f"disable_p2p={disable_p2p} comm_stream={comm_stream}")
+    world, bufs = make_world(num_ranks, max_tokens, hidden, num_experts, disable_p2p)
+    assert bufs[0].runtime.p2p_enabled() == (not disable_p2p)
     world.set_option("comm_stream", comm_stream)     # 1: the reference's arrangement, rounds on a stream of their own
     L = num_experts // num_ranks
     alive = [r for r in range(num_ranks) if r != fail_rank]
