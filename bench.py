@@ -489,8 +489,13 @@ def main():
         "kernels": kernels,
         "consumer": consumer,
         "fused_combine": fused,
+        # `achieved` is priced on the kernel's duration inside the running pipeline (an event pair around it in
+        # every step, which carries 2-5 us of marker overhead); the same kernel launched back to back between
+        # one event pair, the figure a profiler's average duration corresponds to, is reported beside it
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "frac_back_to_back": round(kernels[dom]["bytes"] / kernels[dom]["us_back_to_back"] / 1e3
+                                                / HBM_PEAK_GBPS, 4),
                      "traffic": None if opts else traffic, "traffic_measured_at_commit": None if opts else traffic_at},
     }
     if not args.no_flushed:
