@@ -279,8 +279,9 @@ class _CtypesEventHandle:
 
 
 class _RecvHook:
-    def __init__(self, handle: c_void_p):
+    def __init__(self, handle: c_void_p, world: "World"):
         self._h = handle
+        self._world = world          # the hook enqueues work of its world: keep it alive
 
     def __call__(self) -> None:
         _lib.check(_lib.lib().mc_ep_hook_call(self._h))
@@ -375,7 +376,7 @@ class _CtypesBuffer:
             packed_recv_x_scales_ptr, packed_recv_count_ptr, packed_recv_src_info_ptr,
             packed_recv_layout_range_ptr, int(bool(async_)), int(bool(return_recv_hook)), compute_stream_ptr,
             ctypes.byref(ev), ctypes.byref(hook)))
-        return (_CtypesEventHandle(_handle=ev) if ev else None, _RecvHook(hook) if hook else None)
+        return (_CtypesEventHandle(_handle=ev) if ev else None, _RecvHook(hook, self.world) if hook else None)
 
     def combine(self, x_ptr: int, topk_idx_ptr: int, topk_weights_ptr: int, src_info_ptr: int,
                 layout_range_ptr: int, active_ranks_ptr: int, num_local_experts: int, num_combined_tokens: int,
@@ -388,7 +389,7 @@ class _CtypesBuffer:
             num_local_experts, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
             num_experts, timeout_us, int(bool(zero_copy)), combined_x_ptr, int(bool(async_)),
             int(bool(return_recv_hook)), compute_stream_ptr, ctypes.byref(ev), ctypes.byref(hook)))
-        return (_CtypesEventHandle(_handle=ev) if ev else None, _RecvHook(hook) if hook else None)
+        return (_CtypesEventHandle(_handle=ev) if ev else None, _RecvHook(hook, self.world) if hook else None)
 
 
 if _native is not None:
