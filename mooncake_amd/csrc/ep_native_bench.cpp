@@ -6,12 +6,18 @@
 //     recv_count clear + bf16 dispatch + combine, legacy_buffer_perf.cpp:84-146).
 //
 //   ep_native_bench [--ranks R] [--tokens T] [--hidden H] [--experts E] [--topk K]
-//                   [--bf16] [--warmups W] [--iterations N]
+//                   [--bf16] [--warmups W] [--iterations N] [--per-rank]
 //
-// Exit status 0 means the self-check passed.  Built by `make bench`.
+// With --per-rank it first drives the per-rank Buffer calls (the reference's binding:
+// mc_ep_buffer_dispatch / mc_ep_buffer_combine, one call per rank and collective) in the three
+// completion modes, with one rank a call ahead of the others, and compares the combined rows bit for
+// bit with the same multiply-add chain on the host.
+//
+// Exit status 0 means the self-checks passed.  Built by `make bench`.
 #include <hip/hip_runtime.h>
 
 #include <chrono>
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -42,7 +48,7 @@ namespace {
 
 struct Args {
     int ranks = 32, tokens = 128, hidden = 7168, experts = 256, topk = 8, warmups = 20, iterations = 30;
-    bool fp8 = true;
+    bool fp8 = true, per_rank = false;
 };
 
 Args parse(int argc, char** argv) {
@@ -64,6 +70,7 @@ Args parse(int argc, char** argv) {
         else if (f == "--warmups") a.warmups = value();
         else if (f == "--iterations") a.iterations = value();
         else if (f == "--bf16") a.fp8 = false;
+        else if (f == "--per-rank") a.per_rank = true;
         else {
             std::fprintf(stderr, "unknown flag %s\n", f.c_str());
             std::exit(2);
@@ -109,6 +116,110 @@ std::vector<uint64_t> per_rank(const T* base, size_t stride_elems, int ranks) {
     std::vector<uint64_t> p((size_t)ranks);
     for (int r = 0; r < ranks; ++r) p[(size_t)r] = (uint64_t)(base + (size_t)r * stride_elems);
     return p;
+}
+
+float from_bf16(uint16_t h) {
+    const uint32_t u = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+// What the per-rank self-test works on: per-rank device addresses and the host copies it checks against.
+struct PerRank {
+    int R, T, H, E, K;
+    bool fp8;
+    std::vector<uint64_t> x, idx, w, active, recv, scales, recv16, count, src, range, out;
+    const uint16_t* out_base;
+    const std::vector<uint16_t>* hx;
+    const std::vector<float>* hw;
+};
+
+// One dispatch + combine through the per-rank calls.  mode 0: the caller's stream waits inside the
+// call; 1: async, an event per call; 2: receive hooks.  Rank 0 posts its dispatch first and, with
+// `ahead`, a second one before any other rank has posted its first.
+int per_rank_cycle(std::vector<mc_ep_buffer_t*>& bufs, const PerRank& p, int mode, bool fp8, bool ahead,
+                   hipStream_t stream, std::vector<mc_ep_event_t*>& keep) {
+    const int R = p.R, T = p.T, H = p.H, E = p.E, K = p.K, L = E / R;
+    const uint64_t s = (uint64_t)stream;
+    const int async = mode == 1, hook = mode == 2;
+    HIP_OK(hipMemsetAsync((void*)p.out_base, 0xFF, (size_t)R * T * H * 2, stream));
+    std::vector<mc_ep_event_t*> events;
+    std::vector<mc_ep_hook_t*> hooks;
+    auto post_dispatch = [&](int r) {
+        mc_ep_event_t* ev = nullptr;
+        mc_ep_hook_t* hk = nullptr;
+        EP_OK(mc_ep_buffer_dispatch(bufs[(size_t)r], p.x[(size_t)r], p.idx[(size_t)r], p.active[(size_t)r], T, H, K, T, E,
+                                    -1, fp8 ? 1 : 0, fp8 ? p.recv[(size_t)r] : p.recv16[(size_t)r],
+                                    fp8 ? p.scales[(size_t)r] : 0, p.count[(size_t)r], p.src[(size_t)r],
+                                    p.range[(size_t)r], async, hook, s, &ev, &hk));
+        if ((ev != nullptr) != (async != 0) || (hk != nullptr) != (hook != 0)) {
+            std::fprintf(stderr, "per-rank dispatch: event / hook do not follow the flags\n");
+            std::exit(1);
+        }
+        if (ev) events.push_back(ev);
+        if (hk) hooks.push_back(hk);
+    };
+    const int rounds = ahead ? 2 : 1;
+    for (int j = 0; j < rounds; ++j) post_dispatch(0);
+    if (R > 1) {
+        int dp = -1, cp = -1;
+        EP_OK(mc_ep_buffer_pending_calls(bufs[0], &dp, &cp));
+        if (dp != rounds || cp != 0) {
+            std::fprintf(stderr, "per-rank: rank 0 has %d dispatches pending, expected %d\n", dp, rounds);
+            return 1;
+        }
+        // waiting for a collective that other ranks have not joined is an error, not a hang
+        if (async && mc_ep_event_synchronize(events[0]) != MC_EP_ERR_PENDING) {
+            std::fprintf(stderr, "per-rank: an incomplete round did not report MC_EP_ERR_PENDING\n");
+            return 1;
+        }
+    }
+    for (int j = 0; j < rounds; ++j)
+        for (int r = 1; r < R; ++r) post_dispatch(r);
+    for (mc_ep_hook_t* hk : hooks) EP_OK(mc_ep_hook_call(hk));
+    for (mc_ep_event_t* ev : events) EP_OK(mc_ep_event_current_stream_wait(ev, s));
+
+    // the dispatched rows are the expert outputs (bf16) - fp8 rounds only have their counts checked
+    std::vector<mc_ep_event_t*> cevents;
+    std::vector<mc_ep_hook_t*> chooks;
+    if (!fp8) {
+        for (int r = 0; r < R; ++r) {
+            mc_ep_event_t* ev = nullptr;
+            mc_ep_hook_t* hk = nullptr;
+            EP_OK(mc_ep_buffer_combine(bufs[(size_t)r], p.recv16[(size_t)r], p.idx[(size_t)r], p.w[(size_t)r],
+                                       p.src[(size_t)r], p.range[(size_t)r], p.active[(size_t)r], L, T, H, K, T, E, -1,
+                                       0, p.out[(size_t)r], async, hook, s, &ev, &hk));
+            if (ev) cevents.push_back(ev);
+            if (hk) chooks.push_back(hk);
+        }
+        for (mc_ep_hook_t* hk : chooks) EP_OK(mc_ep_hook_call(hk));
+        for (mc_ep_event_t* ev : cevents) EP_OK(mc_ep_event_synchronize(ev));
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    for (mc_ep_hook_t* hk : hooks) EP_OK(mc_ep_hook_destroy(hk));
+    for (mc_ep_hook_t* hk : chooks) EP_OK(mc_ep_hook_destroy(hk));
+    // events are the caller's to release whenever it likes: main does, after the world is gone
+    keep.insert(keep.end(), events.begin(), events.end());
+    keep.insert(keep.end(), cevents.begin(), cevents.end());
+    if (fp8) return 0;
+
+    // combine of the dispatched rows: fp32 multiply-add chain over k, rounded to bf16 once
+    std::vector<uint16_t> got((size_t)R * T * H);
+    HIP_OK(hipMemcpy(got.data(), p.out_base, got.size() * 2, hipMemcpyDeviceToHost));
+    for (size_t n = 0; n < (size_t)R * T; ++n) {
+        for (int h = 0; h < H; ++h) {
+            const float v = from_bf16((*p.hx)[n * H + h]);
+            float acc = 0.0f;
+            for (int k = 0; k < K; ++k) acc = std::fmaf(v, (*p.hw)[n * K + k], acc);
+            if (got[n * H + h] != to_bf16(acc)) {
+                std::fprintf(stderr, "per-rank mode %d: token %zu element %d is 0x%04x, expected 0x%04x\n", mode, n, h,
+                             got[n * H + h], to_bf16(acc));
+                return 1;
+            }
+        }
+    }
+    return 0;
 }
 
 }  // namespace
@@ -176,6 +287,23 @@ int main(int argc, char** argv) {
     HIP_OK(hipStreamCreate(&stream));
     const uint64_t s = (uint64_t)stream;
 
+    std::vector<mc_ep_event_t*> kept_events;
+    if (a.per_rank) {
+        PerRank p{R, T, H, E, K, a.fp8, px, pidx, pw, pact, precv, pscales, precv16, pcnt, psrc, plr, pout, out, &hx, &hw};
+        std::vector<mc_ep_buffer_t*> bufs((size_t)R, nullptr);
+        const int64_t hint = (int64_t)mc_ep_get_buffer_size_hint(T, H, R, E);
+        for (int r = 0; r < R; ++r) EP_OK(mc_ep_buffer_create(world, r, hint, 0, &bufs[(size_t)r]));
+        for (int mode = 0; mode < 3; ++mode) {
+            for (int ahead = 0; ahead < 2; ++ahead) {
+                if (per_rank_cycle(bufs, p, mode, false, ahead != 0, stream, kept_events)) return 1;
+                if (a.fp8 && per_rank_cycle(bufs, p, mode, true, ahead != 0, stream, kept_events)) return 1;
+            }
+        }
+        for (mc_ep_buffer_t* b : bufs) EP_OK(mc_ep_buffer_destroy(b));
+        std::printf("per-rank calls: 3 completion modes x (in step, rank 0 a call ahead), bf16%s: combined rows equal "
+                    "the host chain\n", a.fp8 ? " and fp8" : "");
+    }
+
     auto dispatch = [&] {
         EP_OK(mc_ep_world_dispatch(world, px.data(), pidx.data(), tokens.data(), H, K, T, E, a.fp8 ? 1 : 0, precv.data(),
                                    a.fp8 ? pscales.data() : nullptr, pcnt.data(), psrc.data(), plr.data(),
@@ -233,6 +361,11 @@ int main(int argc, char** argv) {
                 lr.average_us, lr.min_us, lr.max_us);
 
     EP_OK(mc_ep_world_destroy(world));
+    // an EventHandle may outlive the world whose collective it stands for
+    for (mc_ep_event_t* ev : kept_events) EP_OK(mc_ep_event_destroy(ev));
     HIP_OK(hipStreamDestroy(stream));
+    const void* owned[] = {x, idx, wts, active, recv_x, scales, recv_bf16, expert_x, out, recv_count, src_info, layout_range};
+    for (const void* d : owned)
+        if (d) HIP_OK(hipFree((void*)d));
     return 0;
 }

@@ -132,8 +132,9 @@ def test_ep_benchmark_zero_copy_is_refused_like_the_reference_build_without_it(g
 
 
 def test_native_driver_runs_without_python_in_the_loop(gpu_device):
-    """The C++ driver built from the C header alone: self-check (per-expert row counts against a host count)
-    and both timing loops."""
+    """The C++ driver built from the C header alone: the per-rank Buffer calls in the three completion modes
+    (combined rows against the same multiply-add chain on the host, bit for bit), the whole-world self-check
+    (per-expert row counts against a host count) and both timing loops."""
     import os
     import subprocess
     from mooncake_amd import _lib
@@ -141,11 +142,12 @@ def test_native_driver_runs_without_python_in_the_loop(gpu_device):
     assert os.path.exists(exe), "build it first (make -C mooncake_amd/csrc)"
     announce("native driver")
     for flags in (["--ranks", "4", "--tokens", "32", "--hidden", "1024", "--experts", "16", "--topk", "4",
-                   "--warmups", "2", "--iterations", "4"],
+                   "--warmups", "2", "--iterations", "4", "--per-rank"],
                   ["--ranks", "2", "--tokens", "17", "--hidden", "256", "--experts", "6", "--topk", "3", "--bf16",
-                   "--warmups", "1", "--iterations", "3"]):
+                   "--warmups", "1", "--iterations", "3", "--per-rank"]):
         run = subprocess.run([exe] + flags, capture_output=True, text=True, timeout=100)
         assert run.returncode == 0, run.stderr
         assert "us per step" in run.stdout and "native loop" in run.stdout
+        assert "combined rows equal the host chain" in run.stdout
     bad = subprocess.run([exe, "--ranks", "3", "--experts", "16"], capture_output=True, text=True, timeout=100)
     assert bad.returncode == 2 and "unusable shape" in bad.stderr
