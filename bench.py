@@ -290,11 +290,25 @@ def stream_ceilings(cfg, S, iters):
     src = torch.empty(big, dtype=torch.uint8, device="cuda:0").fill_(3)
     dst = torch.empty(big, dtype=torch.uint8, device="cuda:0")
     res = {}
+
+    def record(name, us, rd, wr):
+        res[name] = {"us": round(us, 2), "read_MB": round(rd / 1e6, 1), "written_MB": round(wr / 1e6, 1),
+                     "GBps": round((rd + wr) / us / 1e3, 1), "pct_of_hbm_peak": round((rd + wr) / us / 1e3 / 80, 2)}
+
     for name, (kind, ub, rd, wr) in mixes.items():
         us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_stream(kind, dst.data_ptr(), src.data_ptr(), ub,
                                                                           stream)), iters)
-        res[name] = {"us": round(us, 2), "read_MB": round(rd / 1e6, 1), "written_MB": round(wr / 1e6, 1),
-                     "GBps": round((rd + wr) / us / 1e3, 1), "pct_of_hbm_peak": round((rd + wr) / us / 1e3 / 80, 2)}
+        record(name, us, rd, wr)
+    del src
+    # the same 8 : 1 gather on the geometry of the packed layout: whole rows at scattered places of
+    # [experts, ranks * max_tokens, hidden] bf16, the valid rows at the start of every expert's block
+    region_rows = cfg.num_ranks * cfg.max_tokens
+    used = max(1, -(-S // cfg.num_experts))
+    layout = torch.empty((cfg.num_experts, region_rows, H), dtype=torch.bfloat16, device="cuda:0")
+    layout[:, :used].fill_(1.0)
+    us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_gather_rows(
+        dst.data_ptr(), layout.data_ptr(), H * 2, N, cfg.num_experts, region_rows, used, stream)), iters)
+    record("gather 8:1 of scattered rows of the packed layout, reduce sized", us, 8 * N * H * 2, N * H * 2)
     return res
 
 
@@ -377,6 +391,10 @@ def main():
             # gather 8:1 sized like the reduce kernel, scatter 1:4 like the fp8 pack kernel, widen 1:2 like cast_back
             for kind, unit_bytes in ((4, N * H * 2), (5, S * H // 8), (3, S * H * 2)):
                 _lib.check(lib.mc_ep_debug_stream(kind, dst.data_ptr(), src.data_ptr(), unit_bytes // 4096 * 4096, stream))
+            # the gather again, on scattered rows of the layout the reduce kernel reads (its expert outputs)
+            _lib.check(lib.mc_ep_debug_gather_rows(dst.data_ptr(), h.expert_out.data_ptr(), H * 2, N, cfg.num_experts,
+                                                   cfg.num_ranks * cfg.max_tokens, max(1, -(-S // cfg.num_experts)),
+                                                   stream))
         torch.cuda.synchronize()
         print(json.dumps({"workload": cfg.name, "kernel_pass": args.kernel_pass}))
         return

@@ -1197,6 +1197,33 @@ __global__ __launch_bounds__(256) void stream_kernel(uint4* __restrict__ dst, co
     }
 }
 
+// The reduce kernel's address pattern without its index loads and arithmetic: every output row of
+// row_units 16-byte units is the xor of 8 whole source rows, and each source row sits at a computed,
+// scattered place of a [regions, region_rows] layout of which the first `used` rows per region are
+// touched, each once (the packed receive layout: a region per expert, valid rows at its start).
+__global__ __launch_bounds__(256) void stream_rows_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                                           int row_units, size_t n, int regions, size_t region_rows,
+                                                           int used) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const size_t ro = i / (size_t)row_units, c = i - ro * (size_t)row_units;
+    uint4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        // a permutation of the regions * used rows (the multiplier is prime), so every row is read once
+        const size_t total = (size_t)regions * (size_t)used;
+        const size_t p = ((ro * 8 + (size_t)k) * 2654435761ull) % total;
+        const size_t region = p % (size_t)regions, rr = p / (size_t)regions;
+        v[k] = load16<true>(src + (region * region_rows + rr) * (size_t)row_units + c);
+    }
+    uint4 a = v[0];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) {
+        a.x ^= v[k].x; a.y ^= v[k].y; a.z ^= v[k].z; a.w ^= v[k].w;
+    }
+    store16<true>(dst + i, a);
+}
+
 __global__ __launch_bounds__(256) void fill_kernel(uint32_t* __restrict__ dst, uint32_t value, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -1504,6 +1531,18 @@ hipError_t launch_stream(int kind, void* dst, const void* src, size_t unit_bytes
         case 4: hipLaunchKernelGGL(stream_kernel<4>, grid, block, 0, stream, d, s, n); break;
         default: hipLaunchKernelGGL(stream_kernel<5>, grid, block, 0, stream, d, s, n); break;
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_stream_rows(void* dst, const void* src, int row_bytes, long long out_rows, int regions,
+                              long long region_rows, int used, hipStream_t stream) {
+    const int row_units = row_bytes / 16;
+    const size_t n = (size_t)out_rows * row_units;
+    if (n == 0) return hipSuccess;
+    const size_t blocks = (n + 255) / 256;
+    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(stream_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src,
+                       row_units, n, regions, (size_t)region_rows, used);
     return hipGetLastError();
 }
 

@@ -1367,7 +1367,9 @@ int mc_ep_event_synchronize(mc_ep_event_t* ev) {
         return MC_EP_OK;
     }
     if (!ev->round || !ev->round->launched) return round_not_ready(ev->round.get());
-    MC_HIP(hipEventSynchronize(ev->round->done));
+    // an async caller's round always has its event; without one, the round's stream says the same
+    if (ev->round->done) MC_HIP(hipEventSynchronize(ev->round->done));
+    else MC_HIP(hipStreamSynchronize(ev->round->launch_stream));
     return MC_EP_OK;
 }
 
@@ -1397,6 +1399,15 @@ int mc_ep_hook_destroy(mc_ep_hook_t* h) {
 int mc_ep_debug_stream(int kind, uint64_t dst_ptr, uint64_t src_ptr, uint64_t unit_bytes, uint64_t stream_ptr) {
     MC_ASSERT(dst_ptr != 0 && src_ptr != 0 && unit_bytes % 16 == 0 && kind >= 0 && kind <= 5);
     MC_HIP(launch_stream(kind, (void*)dst_ptr, (const void*)src_ptr, (size_t)unit_bytes, (hipStream_t)stream_ptr));
+    return MC_EP_OK;
+}
+
+int mc_ep_debug_gather_rows(uint64_t dst_ptr, uint64_t src_ptr, int row_bytes, int64_t out_rows, int regions,
+                            int64_t region_rows, int used, uint64_t stream_ptr) {
+    MC_ASSERT(dst_ptr != 0 && src_ptr != 0 && row_bytes > 0 && row_bytes % 16 == 0 && out_rows >= 0);
+    MC_ASSERT(regions > 0 && used > 0 && region_rows >= used && out_rows < (1ll << 28));
+    MC_HIP(launch_stream_rows((void*)dst_ptr, (const void*)src_ptr, row_bytes, (long long)out_rows, regions,
+                              (long long)region_rows, used, (hipStream_t)stream_ptr));
     return MC_EP_OK;
 }
 
