@@ -30,7 +30,7 @@ int mc_ep_debug_copy(uint64_t dst_ptr, uint64_t src_ptr, uint64_t bytes, uint64_
 int mc_ep_debug_stream(int kind, uint64_t dst_ptr, uint64_t src_ptr, uint64_t unit_bytes, uint64_t stream_ptr);
 
 /* The reduce kernel's address pattern with nothing else: out_rows rows of
- * row_bytes (multiple of 16), each the xor of 8 whole rows at computed,
+ * row_bytes (multiple of 1024), each the xor of 8 whole rows at computed,
  * scattered places of a [regions, region_rows, row_bytes] source of which the
  * first `used` rows of every region are read (the packed layout: a region per
  * expert, its valid rows at the start).  No index loads, no arithmetic. */

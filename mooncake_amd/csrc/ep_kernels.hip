@@ -1206,15 +1206,17 @@ __global__ __launch_bounds__(256) void stream_rows_kernel(uint4* __restrict__ ds
                                                            int used) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    const size_t ro = i / (size_t)row_units, c = i - ro * (size_t)row_units;
+    // a row is a whole number of waves (row_units % 64 == 0), so the row arithmetic is the wave's, not the lane's
+    const uint32_t ro = __builtin_amdgcn_readfirstlane((uint32_t)(i / (size_t)row_units));
+    const size_t c = i - (size_t)ro * (size_t)row_units;
+    const uint32_t total = (uint32_t)regions * (uint32_t)used;
     uint4 v[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         // a permutation of the regions * used rows (the multiplier is prime), so every row is read once
-        const size_t total = (size_t)regions * (size_t)used;
-        const size_t p = ((ro * 8 + (size_t)k) * 2654435761ull) % total;
-        const size_t region = p % (size_t)regions, rr = p / (size_t)regions;
-        v[k] = load16<true>(src + (region * region_rows + rr) * (size_t)row_units + c);
+        const uint32_t p = (uint32_t)(((uint64_t)(ro * 8u + (uint32_t)k) * 2654435761ull) % total);
+        const uint32_t region = p % (uint32_t)regions, rr = p / (uint32_t)regions;
+        v[k] = load16<true>(src + ((size_t)region * region_rows + rr) * (size_t)row_units + c);
     }
     uint4 a = v[0];
 #pragma unroll
@@ -1539,6 +1541,7 @@ hipError_t launch_stream_rows(void* dst, const void* src, int row_bytes, long lo
     const int row_units = row_bytes / 16;
     const size_t n = (size_t)out_rows * row_units;
     if (n == 0) return hipSuccess;
+    if (row_units % 64 != 0 || (long long)regions * used > 0x7fffffffll) return hipErrorInvalidValue;
     const size_t blocks = (n + 255) / 256;
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
     hipLaunchKernelGGL(stream_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src,

@@ -1404,7 +1404,7 @@ int mc_ep_debug_stream(int kind, uint64_t dst_ptr, uint64_t src_ptr, uint64_t un
 
 int mc_ep_debug_gather_rows(uint64_t dst_ptr, uint64_t src_ptr, int row_bytes, int64_t out_rows, int regions,
                             int64_t region_rows, int used, uint64_t stream_ptr) {
-    MC_ASSERT(dst_ptr != 0 && src_ptr != 0 && row_bytes > 0 && row_bytes % 16 == 0 && out_rows >= 0);
+    MC_ASSERT(dst_ptr != 0 && src_ptr != 0 && row_bytes > 0 && row_bytes % 1024 == 0 && out_rows >= 0);
     MC_ASSERT(regions > 0 && used > 0 && region_rows >= used && out_rows < (1ll << 28));
     MC_HIP(launch_stream_rows((void*)dst_ptr, (const void*)src_ptr, row_bytes, (long long)out_rows, regions,
                               (long long)region_rows, used, (hipStream_t)stream_ptr));
