@@ -63,6 +63,10 @@ def parse_args():
     ap.add_argument("--stream-ceilings", action="store_true",
                     help="instead of the workload, time synthetic streams with the data kernels' read : write mixes "
                          "and byte counts (what the memory system gives each mix), and print them as JSON")
+    ap.add_argument("--gather-geometries", action="store_true",
+                    help="instead of the workload, time the 8 : 1 gather of whole scattered rows over several layouts "
+                         "of the same rows (with and without gaps between the experts' blocks) and the sequential "
+                         "gather beside them, and print them as JSON")
     ap.add_argument("--kernel-pass", type=int, default=0, metavar="N",
                     help="instead of timing, run every kernel of the workload (dispatch, cast_back, combine, packed "
                          "combine) and the synthetic streams sized like them N times and exit: the program to put "
@@ -312,6 +316,35 @@ def stream_ceilings(cfg, S, iters):
     return res
 
 
+def gather_geometries(cfg, S, iters):
+    """The scattered-row gather of stream_ceilings over other placements of the same number of rows: is it the
+    gaps between the experts' blocks that cost, or reading whole rows in a scattered order?"""
+    import torch
+    from mooncake_amd import _lib
+    lib = _lib.lib()
+    stream = int(torch.cuda.current_stream().cuda_stream)
+    H, N, E = cfg.hidden, cfg.total_tokens, cfg.num_experts
+    region_rows = cfg.num_ranks * cfg.max_tokens
+    used = max(1, -(-S // E))
+    layout = torch.empty((E, region_rows, H), dtype=torch.bfloat16, device="cuda:0").fill_(1.0)
+    dst = torch.empty(N * H * 2, dtype=torch.uint8, device="cuda:0")
+    res = {}
+    for name, (regions, rows, use) in {
+        "the packed layout (a block per expert, valid rows at its start)": (E, region_rows, used),
+        "the same rows without gaps (one block)": (1, E * used, E * used),
+        "blocks without gaps (experts x valid rows)": (E, used, used),
+        "8 blocks": (8, E * used // 8, E * used // 8),
+        "16 times the blocks, a 16th of the rows each": (E * 16, max(1, region_rows // 16), max(1, used // 16)),
+    }.items():
+        us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_gather_rows(
+            dst.data_ptr(), layout.data_ptr(), H * 2, N, regions, rows, use, stream)), iters)
+        res[name] = {"regions": regions, "region_rows": rows, "used": use, "us": round(us, 2)}
+    us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_stream(4, dst.data_ptr(), layout.data_ptr(),
+                                                                      N * H * 2 // 4096 * 4096, stream)), iters)
+    res["sequential gather 8:1 (no rows)"] = {"us": round(us, 2)}
+    return res
+
+
 def cpu_baseline(cfg, data, bytes_total, budget_s):
     """The oracle (a scalar C restatement, OpenMP over tokens) timed on this
     host's cores on the same workload: whole steps until the budget is spent."""
@@ -371,6 +404,10 @@ def main():
 
     if args.stream_ceilings:
         print(json.dumps({"workload": cfg.name, "stream_ceilings": stream_ceilings(cfg, S, args.kernel_iters)}))
+        return
+
+    if args.gather_geometries:
+        print(json.dumps({"workload": cfg.name, "gather_geometries": gather_geometries(cfg, S, args.kernel_iters)}))
         return
 
     if args.kernel_pass > 0:
