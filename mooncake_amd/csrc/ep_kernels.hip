@@ -82,38 +82,38 @@ __device__ __forceinline__ uint64_t read_lane_u64(uint64_t v, int lane) {
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
+// Every tensor the kernels touch is device memory, but most addresses reach them as integers (rank tables,
+// kernel arguments), which the compiler can only treat as generic pointers: flat loads and stores, which
+// also count as LDS / scalar-memory operations when a wave waits.  These helpers say "global" explicitly.
+#define MCEP_GLOBAL __attribute__((address_space(1)))
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
 template <bool NT>
 __device__ __forceinline__ uint4 load16(const void* p) {
-    if (NT) {
-        const uint32_t* q = (const uint32_t*)p;
-        typedef uint32_t v4 __attribute__((ext_vector_type(4)));
-        v4 r = __builtin_nontemporal_load((const v4*)q);
-        return make_uint4(r.x, r.y, r.z, r.w);
-    }
-    return *(const uint4*)p;
+    const MCEP_GLOBAL u32x4* q = (const MCEP_GLOBAL u32x4*)(uintptr_t)p;
+    const u32x4 r = NT ? __builtin_nontemporal_load(q) : *q;
+    return make_uint4(r.x, r.y, r.z, r.w);
 }
 
 template <bool NT>
 __device__ __forceinline__ void store16(void* p, uint4 v) {
-    if (NT) {
-        typedef uint32_t v4 __attribute__((ext_vector_type(4)));
-        v4 r = {v.x, v.y, v.z, v.w};
-        __builtin_nontemporal_store(r, (v4*)p);
-    } else {
-        *(uint4*)p = v;
-    }
+    MCEP_GLOBAL u32x4* q = (MCEP_GLOBAL u32x4*)(uintptr_t)p;
+    const u32x4 r = {v.x, v.y, v.z, v.w};
+    if (NT) __builtin_nontemporal_store(r, q);
+    else *q = r;
 }
 
 template <bool NT>
 __device__ __forceinline__ void store8(void* p, uint2 v) {
-    if (NT) {
-        typedef uint32_t v2 __attribute__((ext_vector_type(2)));
-        v2 r = {v.x, v.y};
-        __builtin_nontemporal_store(r, (v2*)p);
-    } else {
-        *(uint2*)p = v;
-    }
+    MCEP_GLOBAL u32x2* q = (MCEP_GLOBAL u32x2*)(uintptr_t)p;
+    const u32x2 r = {v.x, v.y};
+    if (NT) __builtin_nontemporal_store(r, q);
+    else *q = r;
 }
+
+__device__ __forceinline__ float load_f32(uint64_t addr) { return *(const MCEP_GLOBAL float*)(uintptr_t)addr; }
+__device__ __forceinline__ int load_i32(uint64_t addr) { return *(const MCEP_GLOBAL int*)(uintptr_t)addr; }
 
 // ---------------------------------------------------------------------------
 // table writer: the host's per-rank pointer table travels in kernel arguments
@@ -697,7 +697,7 @@ __device__ __forceinline__ DirectRow direct_row(const uint64_t* __restrict__ tbl
                                                 int lane) {
     const int RM = R * max_tokens;
     const int L = E / R;
-    const int32_t* active = (const int32_t*)tbl[CF_ACTIVE * R + r];
+    const uint64_t active = tbl[CF_ACTIVE * R + r];
     const int sr = sc.selrow[((int64_t)r * max_tokens + t) * K + (lane < K ? lane : 0)];
     DirectRow d;
     d.has = lane < K && sr >= 0;
@@ -706,8 +706,13 @@ __device__ __forceinline__ DirectRow direct_row(const uint64_t* __restrict__ tbl
     d.q = d.e / L;
     d.le = d.e - d.q * L;
     d.base = rank_ptr(tbl, x, CF_X, R, d.q);
-    d.live = active[d.q];
     d.grow = (int64_t)d.le * RM + d.slot;
+    // `live` is asked for last, behind whatever the base address had to wait for (a table entry when the
+    // ranks' tensors are not evenly spaced): loads complete in order for a waiting wave, so a load issued
+    // before that wait would be waited for as well, ahead of the payload
+    int q_late = d.q;
+    asm volatile("" : "+v"(q_late) : "v"((uint32_t)d.base), "v"((uint32_t)(d.base >> 32)));
+    d.live = load_i32(active + (uint64_t)q_late * 4);
     return d;
 }
 
@@ -739,8 +744,8 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
     if (DIRECT) {
         // the caller's top-k rows exist only for t < T
         if (t >= T) return;
-        const float* w_row = (const float*)rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (int64_t)t * K;
-        const float wl = w_row[lane < K ? lane : 0];
+        const uint64_t w_row = rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (uint64_t)((int64_t)t * K) * 4;
+        const float wl = load_f32(w_row + (uint64_t)(lane < K ? lane : 0) * 4);
         const DirectRow d = direct_row(tbl, sc, cs.x, R, E, K, max_tokens, r, t, lane);
         if (d.has && d.base != 0) {
             src = d.base + (uint64_t)d.grow * (uint64_t)H * 2;
@@ -885,8 +890,8 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
         bool ok = false;
         float wl = 0.0f;
         if (DIRECT) {
-            const float* w_row = (const float*)rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (int64_t)t * K;
-            wl = w_row[lane < K ? lane : 0];
+            const uint64_t w_row = rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (uint64_t)((int64_t)t * K) * 4;
+            wl = load_f32(w_row + (uint64_t)(lane < K ? lane : 0) * 4);
             const DirectRow d = direct_row(tbl, sc, cs.x, R, E, K, max_tokens, r, t, lane);
             ok = d.has;
             e = d.e;
@@ -926,12 +931,11 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
         const uint64_t p = read_lane_u64(src, k);
-        fk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), k));
         v[k] = load16<true>((const void*)(p + poff));
         if (FP8) {
             const uint64_t sp = read_lane_u64(ssrc, k);
             const int st = __builtin_amdgcn_readlane(sstride, k);
-            sv[k] = *(const float*)(sp + (int64_t)group * st);
+            sv[k] = load_f32(sp + (uint64_t)((int64_t)group * st));
         } else {
             sv[k] = 1.0f;
         }
@@ -939,8 +943,12 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
 
     // a row of a rank the token's owner sees as inactive was fetched before that was known: drop it
     if (DIRECT && live == 0) w = 0.0f;
+    // the expert's factor was loaded behind the row table, like `live`: looked at only now, when the payload
+    // loads are on their way
+    asm volatile("" : "+v"(f));
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
+        fk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), k));
         wk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k));
         if (DIRECT && __builtin_amdgcn_readlane(live, k) == 0) {
             v[k] = make_uint4(0, 0, 0, 0);
