@@ -24,7 +24,15 @@ _ZERO_COPY_COMBINE_UNSUPPORTED = (
 )
 
 
+# torch.cuda.current_stream() builds a Stream object behind several Python-level device look-ups (about 4 us
+# a call, twice per dispatch or combine); torch's own raw-stream query gives the same address directly
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _native_current_stream_ptr() -> int:
+    if _raw_stream is not None and _raw_device is not None:
+        return int(_raw_stream(_raw_device()))
     return int(torch.cuda.current_stream().cuda_stream)
 
 

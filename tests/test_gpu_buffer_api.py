@@ -294,3 +294,16 @@ def test_host_assertions_and_unsupported(gpu_device):
         buf.get_next_combine_buffer(handle)
     assert buf.runtime.ibgda_disabled() and buf.runtime.use_fast_path() and not buf.runtime.is_roce()
     assert buf.runtime.get_local_qpns() == [] and buf.runtime.get_mr_info() == (0, 0)
+
+
+def test_the_buffer_sees_the_callers_current_stream(gpu_device):
+    """Buffer.dispatch / combine run on torch's current stream (reference: mooncake_ep_buffer.py:488-507 passes
+    torch.cuda.current_stream().cuda_stream); the wrapper's shortcut to that address must follow stream contexts."""
+    from mooncake_amd import mooncake_ep_buffer as mod
+    announce("current stream lookup")
+    assert mod._native_current_stream_ptr() == torch.cuda.current_stream().cuda_stream
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        assert mod._native_current_stream_ptr() == side.cuda_stream
+        assert mod._native_current_stream_ptr() == torch.cuda.current_stream().cuda_stream
+    assert mod._native_current_stream_ptr() == torch.cuda.current_stream().cuda_stream
