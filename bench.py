@@ -313,6 +313,13 @@ def stream_ceilings(cfg, S, iters):
     us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_gather_rows(
         dst.data_ptr(), layout.data_ptr(), H * 2, N, cfg.num_experts, region_rows, used, stream)), iters)
     record("gather 8:1 of scattered rows of the packed layout, reduce sized", us, 8 * N * H * 2, N * H * 2)
+    # and the 1 : 4 scatter on the geometry of the fp8 layout: every source row read once, written (at half its
+    # size) to 8 whole rows at scattered places of [experts, ranks * max_tokens, hidden] bytes
+    layout8 = layout.view(torch.uint8)[: cfg.num_experts * region_rows * H]
+    src16 = torch.empty(N * H * 2, dtype=torch.uint8, device="cuda:0").fill_(3)
+    us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_scatter_rows(
+        layout8.data_ptr(), src16.data_ptr(), H, N, cfg.num_experts, region_rows, used, stream)), iters)
+    record("scatter 1:4 to scattered rows of the fp8 layout, fp8-pack sized", us, N * H * 2, 8 * N * H)
     return res
 
 

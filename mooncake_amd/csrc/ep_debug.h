@@ -37,6 +37,14 @@ int mc_ep_debug_stream(int kind, uint64_t dst_ptr, uint64_t src_ptr, uint64_t un
 int mc_ep_debug_gather_rows(uint64_t dst_ptr, uint64_t src_ptr, int row_bytes, int64_t out_rows, int regions,
                             int64_t region_rows, int used, uint64_t stream_ptr);
 
+/* The fp8 pack kernel's address pattern with nothing else: in_rows source rows
+ * of 2 * row_bytes, read once, folded to row_bytes (multiple of 1024) and
+ * written to 8 whole rows at computed, scattered places of a
+ * [regions, region_rows, row_bytes] destination (the first `used` rows of every
+ * region, each written once). */
+int mc_ep_debug_scatter_rows(uint64_t dst_ptr, uint64_t src_ptr, int row_bytes, int64_t in_rows, int regions,
+                             int64_t region_rows, int used, uint64_t stream_ptr);
+
 #ifdef __cplusplus
 }
 #endif

@@ -178,6 +178,9 @@ hipError_t launch_stream(int kind, void* dst, const void* src, size_t unit_bytes
 // out_rows rows, each the xor of 8 rows scattered over a [regions, region_rows] layout (see stream_rows_kernel)
 hipError_t launch_stream_rows(void* dst, const void* src, int row_bytes, long long out_rows, int regions,
                               long long region_rows, int used, hipStream_t stream);
+// in_rows rows of 2 * row_bytes, each folded to row_bytes and written to 8 scattered rows (see stream_rows_scatter_kernel)
+hipError_t launch_stream_rows_scatter(void* dst, const void* src, int row_bytes, long long in_rows, int regions,
+                                      long long region_rows, int used, hipStream_t stream);
 // zero `words` 32-bit words at each of n_ptrs device addresses (host array), one launch per kTableChunk addresses
 hipError_t launch_clear_words(const uint64_t* h_ptrs, int n_ptrs, int words, hipStream_t stream);
 hipError_t launch_fill_u32(void* dst, uint32_t value, size_t words, hipStream_t stream);

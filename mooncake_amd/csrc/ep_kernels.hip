@@ -1234,6 +1234,27 @@ __global__ __launch_bounds__(256) void stream_rows_kernel(uint4* __restrict__ ds
     store16<true>(dst + i, a);
 }
 
+// The fp8 pack kernel's address pattern alone: every source row of 2 * row_units units is read once,
+// folded to row_units units and written to 8 whole rows at computed, scattered places of a
+// [regions, region_rows] layout (the first `used` rows of every region, each written once).
+__global__ __launch_bounds__(256) void stream_rows_scatter_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                                                   int row_units, size_t n, int regions,
+                                                                   size_t region_rows, int used) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t ri = __builtin_amdgcn_readfirstlane((uint32_t)(i / (size_t)row_units));
+    const size_t c = i - (size_t)ri * (size_t)row_units;
+    const uint32_t total = (uint32_t)regions * (uint32_t)used;
+    const uint4 a = load16<true>(src + 2 * i), b = load16<true>(src + 2 * i + 1);
+    const uint4 o = make_uint4(a.x ^ b.x, a.y ^ b.y, a.z ^ b.z, a.w ^ b.w);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint32_t p = (uint32_t)(((uint64_t)(ri * 8u + (uint32_t)k) * 2654435761ull) % total);
+        const uint32_t region = p % (uint32_t)regions, rr = p / (uint32_t)regions;
+        store16<false>(dst + ((size_t)region * region_rows + rr) * (size_t)row_units + c, o);
+    }
+}
+
 __global__ __launch_bounds__(256) void fill_kernel(uint32_t* __restrict__ dst, uint32_t value, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -1554,6 +1575,19 @@ hipError_t launch_stream_rows(void* dst, const void* src, int row_bytes, long lo
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
     hipLaunchKernelGGL(stream_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src,
                        row_units, n, regions, (size_t)region_rows, used);
+    return hipGetLastError();
+}
+
+hipError_t launch_stream_rows_scatter(void* dst, const void* src, int row_bytes, long long in_rows, int regions,
+                                      long long region_rows, int used, hipStream_t stream) {
+    const int row_units = row_bytes / 16;
+    const size_t n = (size_t)in_rows * row_units;
+    if (n == 0) return hipSuccess;
+    if (row_units % 64 != 0 || (long long)regions * used > 0x7fffffffll) return hipErrorInvalidValue;
+    const size_t blocks = (n + 255) / 256;
+    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(stream_rows_scatter_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)dst,
+                       (const uint4*)src, row_units, n, regions, (size_t)region_rows, used);
     return hipGetLastError();
 }
 

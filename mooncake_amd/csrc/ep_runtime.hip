@@ -1411,6 +1411,15 @@ int mc_ep_debug_gather_rows(uint64_t dst_ptr, uint64_t src_ptr, int row_bytes, i
     return MC_EP_OK;
 }
 
+int mc_ep_debug_scatter_rows(uint64_t dst_ptr, uint64_t src_ptr, int row_bytes, int64_t in_rows, int regions,
+                             int64_t region_rows, int used, uint64_t stream_ptr) {
+    MC_ASSERT(dst_ptr != 0 && src_ptr != 0 && row_bytes > 0 && row_bytes % 1024 == 0 && in_rows >= 0);
+    MC_ASSERT(regions > 0 && used > 0 && region_rows >= used && in_rows < (1ll << 28));
+    MC_HIP(launch_stream_rows_scatter((void*)dst_ptr, (const void*)src_ptr, row_bytes, (long long)in_rows, regions,
+                                      (long long)region_rows, used, (hipStream_t)stream_ptr));
+    return MC_EP_OK;
+}
+
 int mc_ep_debug_copy(uint64_t dst_ptr, uint64_t src_ptr, uint64_t bytes, uint64_t stream_ptr) {
     MC_ASSERT(dst_ptr != 0 && src_ptr != 0 && bytes % 16 == 0);
     MC_HIP(launch_copy((void*)dst_ptr, (const void*)src_ptr, (size_t)bytes, (hipStream_t)stream_ptr));
