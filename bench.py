@@ -436,9 +436,13 @@ def main():
             for kind, unit_bytes in ((4, N * H * 2), (5, S * H // 8), (3, S * H * 2)):
                 _lib.check(lib.mc_ep_debug_stream(kind, dst.data_ptr(), src.data_ptr(), unit_bytes // 4096 * 4096, stream))
             # the gather again, on scattered rows of the layout the reduce kernel reads (its expert outputs)
+            used = max(1, -(-S // cfg.num_experts))
             _lib.check(lib.mc_ep_debug_gather_rows(dst.data_ptr(), h.expert_out.data_ptr(), H * 2, N, cfg.num_experts,
-                                                   cfg.num_ranks * cfg.max_tokens, max(1, -(-S // cfg.num_experts)),
-                                                   stream))
+                                                   cfg.num_ranks * cfg.max_tokens, used, stream))
+            # and the scatter on scattered rows of a layout shaped like the fp8 payload (the expert outputs' memory,
+            # refilled by the next round's cast_back)
+            _lib.check(lib.mc_ep_debug_scatter_rows(h.expert_out.data_ptr(), src.data_ptr(), H, N, cfg.num_experts,
+                                                    cfg.num_ranks * cfg.max_tokens, used, stream))
         torch.cuda.synchronize()
         print(json.dumps({"workload": cfg.name, "kernel_pass": args.kernel_pass}))
         return
