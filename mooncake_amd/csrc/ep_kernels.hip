@@ -728,7 +728,7 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
                                                       const CombineRoute* __restrict__ routes, uint32_t stamp,
                                                       RoutingScratch sc, CombineSource cs,
                                                       const void* __restrict__ zero_row, int R, int E, int K,
-                                                      int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
+                                                      int max_tokens, int H, int slabs, int Tgrid,
                                                       int total_tasks) {
     const int lane = wave_lane();
     const int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
@@ -857,7 +857,7 @@ __global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __re
                                                              RoutingScratch sc, CombineSource cs,
                                                              const void* __restrict__ zero_row,
                                                              const float* __restrict__ factor, int R, int E, int K,
-                                                             int max_tokens, int H, UnitPlan up, int slabs, int Tgrid,
+                                                             int max_tokens, int H, int slabs, int Tgrid,
                                                              int group_blocks) {
     constexpr int kSlab = FP8 ? 1024 : 512;
     constexpr int kLaneElems = kSlab / 64;
@@ -1438,7 +1438,7 @@ static hipError_t launch_reduce_t(const ReduceLaunch& rl, const Dims& d, const T
 #define MCEP_REDUCE(A, B)                                                                                        \
     hipLaunchKernelGGL((reduce_kernel<KMAX, CH, A, B, DIRECT>), dim3(blocks), dim3(wpb * 64), 0, stream, rl.d_tbl, \
                        rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d.R, d.E, d.K, d.max_tokens, d.H,    \
-                       d.plan, slabs, d.Tgrid, (int)total)
+                       slabs, d.Tgrid, (int)total)
     if (ntl && nts) MCEP_REDUCE(true, true);
     else if (ntl) MCEP_REDUCE(true, false);
     else if (nts) MCEP_REDUCE(false, true);
@@ -1484,7 +1484,7 @@ static hipError_t launch_reduce_packed_t(const ReduceLaunch& rl, const float* d_
     if (blocks > 0x7fffffffll) return hipErrorInvalidValue;
     hipLaunchKernelGGL((reduce_packed_kernel<KMAX, FP8, FACTOR, DIRECT>), dim3((unsigned)blocks), dim3(wpb * 64), 0,
                        stream, rl.d_tbl, rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d_factor, d.R, d.E, d.K,
-                       d.max_tokens, d.H, d.plan, slabs, d.Tgrid, group_blocks);
+                       d.max_tokens, d.H, slabs, d.Tgrid, group_blocks);
     return hipGetLastError();
 }
 

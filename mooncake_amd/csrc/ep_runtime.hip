@@ -174,7 +174,6 @@ struct mc_ep_world {
         int hidden = 0, num_topk = 0, max_tokens = 0, num_experts = 0;
         std::vector<uint64_t> topk_idx, recv_x, src_info, layout_range;
         std::vector<int32_t> num_tokens;
-        UnitPlan plan;                            // how its routing state is laid out
         bool data_done = false;                   // its pack phase has been launched too (and did not fail)
         bool captured = false;                    // recorded into a graph, and which capture
         unsigned long long capture_id = 0;
@@ -544,7 +543,6 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
             ld.src_info.assign(src_info, src_info + R);
             ld.layout_range.assign(layout_range, layout_range + R);
             ld.num_tokens.assign(num_tokens, num_tokens + R);
-            ld.plan = d.plan;
             ld.captured = cap.active;
             ld.capture_id = cap.id;
             ld.data_done = false;
@@ -607,7 +605,6 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     const uint64_t* d_tbl = nullptr;
     if (int rc = upload_table(w, 1, tbl, cap, stream, &d_tbl)) return rc;
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
-    d.plan = w->last.plan;   // read only when the last dispatch's routing state is reused
 
     // Is this the handle (and the routing input) of the last dispatch?  Then the
     // packed row of every selection is already known on the device.  Like the
