@@ -13,8 +13,16 @@
  * ("Failed: Assertion error file:line 'cond'", mooncake_ep_exception.cuh:12-45)
  * where this ABI returns MC_EP_ERR_ASSERT with the same condition text.
  *
- * Not thread-safe per object, like the reference
- * (mooncake_ep_buffer.cpp:215-218): drive one world from one thread.  The
+ * Threads: the library's host bookkeeping sits behind one process-wide lock,
+ * so any thread may call any function; a call holds the lock while it records
+ * arguments and enqueues kernels, never while it waits for the GPU.  What the
+ * lock cannot give is order: calls of one rank must come from one thread at a
+ * time (the reference's buffer is not thread-safe either,
+ * mooncake_ep_buffer.cpp:215-218), and with one driver thread for all ranks a
+ * per-rank call returns before its collective is complete (see
+ * mc_ep_buffer_dispatch).  A thread per rank, each using its results as soon
+ * as its call returns like a process of the reference, sets the option
+ * "blocking".  The
  * calls of one world share its scratch (rank tables, routing state, staged
  * scales), so the library serialises them across streams: a call on another
  * stream than the world's previous call first waits for what that stream
@@ -91,7 +99,13 @@ int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
  * (mooncake_ep_kernel.cu:184, :252), which differ in the last bit of a scale
  * for about a quarter of all groups; "comm_stream": 1 runs every per-rank
  * collective on the world's communication stream as the reference does, 0
- * (default) on the callers' stream when they all share one). */
+ * (default) on the callers' stream when they all share one; "blocking": 1
+ * makes mc_ep_buffer_dispatch / mc_ep_buffer_combine return only when the
+ * call's round has been launched - by the thread whose call completed it - so
+ * that work the caller enqueues next on its stream is ordered behind the
+ * round, which is what a thread per rank needs; a call that has waited
+ * "block_timeout_ms" (default 30000) for its peers fails with
+ * MC_EP_ERR_PENDING and stays posted). */
 int mc_ep_world_set_option(mc_ep_world_t* world, const char* name, int value);
 int mc_ep_world_get_option(const mc_ep_world_t* world, const char* name, int* value);
 

@@ -142,6 +142,8 @@ struct Tuning {
     int combine_nt = 3;        // bit 0: streaming loads, bit 1: streaming stores
     int routing_sum = 1;       // allow the summed routing plan (see UnitPlan) where the shape permits
     int comm_stream = 0;       // 1: per-rank rounds always run on the world's communication stream
+    int blocking = 0;          // 1: a per-rank call returns only when its round has been launched (a thread per rank)
+    int block_timeout_ms = 30000;   // how long such a call waits for its peers before it fails
 };
 
 // Chooses the unit plan for a shape (summed when allowed, the shape permits and there are tokens).

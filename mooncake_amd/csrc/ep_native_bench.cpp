@@ -11,7 +11,8 @@
 // With --per-rank it first drives the per-rank Buffer calls (the reference's binding:
 // mc_ep_buffer_dispatch / mc_ep_buffer_combine, one call per rank and collective) in the three
 // completion modes, with one rank a call ahead of the others, and compares the combined rows bit for
-// bit with the same multiply-add chain on the host.
+// bit with the same multiply-add chain on the host; then once more with a thread per rank, each on a
+// stream of its own, under the world's option "blocking".
 //
 // Exit status 0 means the self-checks passed.  Built by `make bench`.
 #include <hip/hip_runtime.h>
@@ -23,6 +24,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "mooncake_ep_hip.h"
@@ -135,6 +137,26 @@ struct PerRank {
     const std::vector<float>* hw;
 };
 
+// Compares the combined rows on the device with the host's chain: fp32 multiply-add over k, one rounding.
+int check_combined(const PerRank& p, const char* what) {
+    const int R = p.R, T = p.T, H = p.H, K = p.K;
+    std::vector<uint16_t> got((size_t)R * T * H);
+    HIP_OK(hipMemcpy(got.data(), p.out_base, got.size() * 2, hipMemcpyDeviceToHost));
+    for (size_t n = 0; n < (size_t)R * T; ++n) {
+        for (int h = 0; h < H; ++h) {
+            const float v = from_bf16((*p.hx)[n * H + h]);
+            float acc = 0.0f;
+            for (int k = 0; k < K; ++k) acc = std::fmaf(v, (*p.hw)[n * K + k], acc);
+            if (got[n * H + h] != to_bf16(acc)) {
+                std::fprintf(stderr, "%s: token %zu element %d is 0x%04x, expected 0x%04x\n", what, n, h,
+                             got[n * H + h], to_bf16(acc));
+                return 1;
+            }
+        }
+    }
+    return 0;
+}
+
 // One dispatch + combine through the per-rank calls.  mode 0: the caller's stream waits inside the
 // call; 1: async, an event per call; 2: receive hooks.  Rank 0 posts its dispatch first and, with
 // `ahead`, a second one before any other rank has posted its first.
@@ -204,22 +226,66 @@ int per_rank_cycle(std::vector<mc_ep_buffer_t*>& bufs, const PerRank& p, int mod
     keep.insert(keep.end(), cevents.begin(), cevents.end());
     if (fp8) return 0;
 
-    // combine of the dispatched rows: fp32 multiply-add chain over k, rounded to bf16 once
-    std::vector<uint16_t> got((size_t)R * T * H);
-    HIP_OK(hipMemcpy(got.data(), p.out_base, got.size() * 2, hipMemcpyDeviceToHost));
-    for (size_t n = 0; n < (size_t)R * T; ++n) {
-        for (int h = 0; h < H; ++h) {
-            const float v = from_bf16((*p.hx)[n * H + h]);
-            float acc = 0.0f;
-            for (int k = 0; k < K; ++k) acc = std::fmaf(v, (*p.hw)[n * K + k], acc);
-            if (got[n * H + h] != to_bf16(acc)) {
-                std::fprintf(stderr, "per-rank mode %d: token %zu element %d is 0x%04x, expected 0x%04x\n", mode, n, h,
-                             got[n * H + h], to_bf16(acc));
-                return 1;
+    char what[32];
+    std::snprintf(what, sizeof(what), "per-rank mode %d", mode);
+    return check_combined(p, what);
+}
+
+// A thread per rank, as a process per rank of the reference: each makes its own calls on its own stream
+// and waits for its own stream only.  With the world's option "blocking" a call returns when the
+// collective has been launched, so the stream order of the caller is enough.
+int thread_per_rank(mc_ep_world_t* world, std::vector<mc_ep_buffer_t*>& bufs, const PerRank& p, int steps) {
+    const int R = p.R, T = p.T, H = p.H, E = p.E, K = p.K, L = E / R;
+    EP_OK(mc_ep_world_set_option(world, "blocking", 1));
+    HIP_OK(hipMemset((void*)p.out_base, 0xFF, (size_t)R * T * H * 2));
+    std::vector<int> failed((size_t)R, 0);
+    std::vector<std::thread> threads;
+    for (int r = 0; r < R; ++r) {
+        threads.emplace_back([&, r] {
+            hipStream_t mine;
+            if (hipStreamCreateWithFlags(&mine, hipStreamNonBlocking) != hipSuccess) {
+                failed[(size_t)r] = 1;
+                return;
             }
-        }
+            const uint64_t s = (uint64_t)mine;
+            for (int j = 0; j < steps && !failed[(size_t)r]; ++j) {
+                const int mode = j % 3;   // default, async, hook in turn: every rank the same mode per step
+                mc_ep_event_t* ev = nullptr;
+                mc_ep_hook_t* hk = nullptr;
+                int rc = mc_ep_buffer_dispatch(bufs[(size_t)r], p.x[(size_t)r], p.idx[(size_t)r], p.active[(size_t)r],
+                                               T, H, K, T, E, -1, 0, p.recv16[(size_t)r], 0, p.count[(size_t)r],
+                                               p.src[(size_t)r], p.range[(size_t)r], mode == 1, mode == 2, s, &ev, &hk);
+                if (rc == MC_EP_OK && ev) rc = mc_ep_event_current_stream_wait(ev, s);
+                if (rc == MC_EP_OK && hk) rc = mc_ep_hook_call(hk);
+                mc_ep_event_destroy(ev);
+                mc_ep_hook_destroy(hk);
+                ev = nullptr;
+                hk = nullptr;
+                if (rc == MC_EP_OK)
+                    rc = mc_ep_buffer_combine(bufs[(size_t)r], p.recv16[(size_t)r], p.idx[(size_t)r], p.w[(size_t)r],
+                                              p.src[(size_t)r], p.range[(size_t)r], p.active[(size_t)r], L, T, H, K, T,
+                                              E, -1, 0, p.out[(size_t)r], mode == 1, mode == 2, s, &ev, &hk);
+                if (rc == MC_EP_OK && ev) rc = mc_ep_event_current_stream_wait(ev, s);
+                if (rc == MC_EP_OK && hk) rc = mc_ep_hook_call(hk);
+                mc_ep_event_destroy(ev);
+                mc_ep_hook_destroy(hk);
+                if (rc != MC_EP_OK) {
+                    std::fprintf(stderr, "rank %d step %d: %s\n", r, j, mc_ep_last_error());
+                    failed[(size_t)r] = 1;
+                }
+                // the next step's dispatch rewrites what this step's combine reads: a rank must not run
+                // ahead of its own stream, exactly as with the reference's buffers
+                if (hipStreamSynchronize(mine) != hipSuccess) failed[(size_t)r] = 1;
+            }
+            (void)hipStreamDestroy(mine);
+        });
     }
-    return 0;
+    for (auto& t : threads) t.join();
+    EP_OK(mc_ep_world_set_option(world, "blocking", 0));
+    for (int r = 0; r < R; ++r)
+        if (failed[(size_t)r]) return 1;
+    HIP_OK(hipDeviceSynchronize());
+    return check_combined(p, "thread per rank");
 }
 
 }  // namespace
@@ -299,9 +365,10 @@ int main(int argc, char** argv) {
                 if (a.fp8 && per_rank_cycle(bufs, p, mode, true, ahead != 0, stream, kept_events)) return 1;
             }
         }
+        if (thread_per_rank(world, bufs, p, 6)) return 1;
         for (mc_ep_buffer_t* b : bufs) EP_OK(mc_ep_buffer_destroy(b));
-        std::printf("per-rank calls: 3 completion modes x (in step, rank 0 a call ahead), bf16%s: combined rows equal "
-                    "the host chain\n", a.fp8 ? " and fp8" : "");
+        std::printf("per-rank calls: 3 completion modes x (in step, rank 0 a call ahead), bf16%s, and a thread per "
+                    "rank: combined rows equal the host chain\n", a.fp8 ? " and fp8" : "");
     }
 
     auto dispatch = [&] {

@@ -49,6 +49,7 @@ using I32s = std::vector<int32_t>;
 struct World {
     mc_ep_world_t* h = nullptr;
     int num_ranks = 0;
+    bool blocking = false;   // option "blocking": per-rank calls wait for their peers, so they must not hold the GIL
     explicit World(int n) : num_ranks(n) { check(mc_ep_world_create(n, &h)); }
     World(const World&) = delete;
     World& operator=(const World&) = delete;
@@ -105,6 +106,14 @@ CallResult wrap(mc_ep_event_t* ev, mc_ep_hook_t* hook, const WorldPtr& world) {
     return r;
 }
 
+// A call that may wait for other Python threads (one per rank, option "blocking") gives up the GIL for
+// its duration; the library reports its failure per thread, so the error text is still this call's.
+template <typename F>
+int without_gil(F&& f) {
+    py::gil_scoped_release release;
+    return f();
+}
+
 // MooncakeEpBuffer, mooncake_ep_buffer.h:66-194
 struct Buffer {
     mc_ep_buffer_t* h = nullptr;
@@ -129,11 +138,14 @@ struct Buffer {
                         uint64_t compute_stream_ptr) {
         mc_ep_event_t* ev = nullptr;
         mc_ep_hook_t* hook = nullptr;
-        check(mc_ep_buffer_dispatch(h, x_ptr, topk_idx_ptr, active_ranks_ptr, num_tokens, hidden, num_topk,
-                                    num_max_dispatch_tokens_per_rank, num_experts, timeout_us, use_fp8 ? 1 : 0,
-                                    packed_recv_x_ptr, packed_recv_x_scales_ptr, packed_recv_count_ptr,
-                                    packed_recv_src_info_ptr, packed_recv_layout_range_ptr, async ? 1 : 0,
-                                    return_recv_hook ? 1 : 0, compute_stream_ptr, &ev, &hook));
+        const auto call = [&] {
+            return mc_ep_buffer_dispatch(h, x_ptr, topk_idx_ptr, active_ranks_ptr, num_tokens, hidden, num_topk,
+                                         num_max_dispatch_tokens_per_rank, num_experts, timeout_us, use_fp8 ? 1 : 0,
+                                         packed_recv_x_ptr, packed_recv_x_scales_ptr, packed_recv_count_ptr,
+                                         packed_recv_src_info_ptr, packed_recv_layout_range_ptr, async ? 1 : 0,
+                                         return_recv_hook ? 1 : 0, compute_stream_ptr, &ev, &hook);
+        };
+        check(world->blocking ? without_gil(call) : call());
         return wrap(ev, hook, world);
     }
 
@@ -144,11 +156,14 @@ struct Buffer {
                        bool return_recv_hook, uint64_t compute_stream_ptr) {
         mc_ep_event_t* ev = nullptr;
         mc_ep_hook_t* hook = nullptr;
-        check(mc_ep_buffer_combine(h, x_ptr, topk_idx_ptr, topk_weights_ptr, src_info_ptr, layout_range_ptr,
-                                   active_ranks_ptr, num_local_experts, num_combined_tokens, hidden, num_topk,
-                                   num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy ? 1 : 0,
-                                   combined_x_ptr, async ? 1 : 0, return_recv_hook ? 1 : 0, compute_stream_ptr, &ev,
-                                   &hook));
+        const auto call = [&] {
+            return mc_ep_buffer_combine(h, x_ptr, topk_idx_ptr, topk_weights_ptr, src_info_ptr, layout_range_ptr,
+                                        active_ranks_ptr, num_local_experts, num_combined_tokens, hidden, num_topk,
+                                        num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy ? 1 : 0,
+                                        combined_x_ptr, async ? 1 : 0, return_recv_hook ? 1 : 0, compute_stream_ptr,
+                                        &ev, &hook);
+        };
+        check(world->blocking ? without_gil(call) : call());
         return wrap(ev, hook, world);
     }
 
@@ -279,7 +294,10 @@ PYBIND11_MODULE(_ep, m) {
              [](World& w, int rank, bool silent) { check(mc_ep_world_set_rank_silent(w.h, rank, silent ? 1 : 0)); },
              py::arg("rank"), py::arg("silent") = true)
         .def("set_option",
-             [](World& w, const std::string& name, int value) { check(mc_ep_world_set_option(w.h, name.c_str(), value)); })
+             [](World& w, const std::string& name, int value) {
+                 check(mc_ep_world_set_option(w.h, name.c_str(), value));
+                 if (name == "blocking") w.blocking = value != 0;
+             })
         .def("get_option",
              [](const World& w, const std::string& name) {
                  int v = 0;

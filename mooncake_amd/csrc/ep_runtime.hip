@@ -8,11 +8,14 @@
 
 #include <hip/hip_runtime.h>
 
+#include <chrono>
+#include <condition_variable>
 #include <cstdio>
 #include <cstring>
 #include <deque>
 #include <functional>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -35,6 +38,15 @@ constexpr int kMaxDevices = 64;
 unsigned char* g_scratch_ptr[kMaxDevices] = {};
 
 thread_local std::string g_last_error;
+
+// One lock for the host bookkeeping of every world, buffer, round, event and hook of the process (an
+// EventHandle may outlive its world, so the lock cannot live in the world): entry points take it for as
+// long as they touch that state and enqueue work, never while they wait for the GPU.  g_round_cv is
+// signalled whenever a round has been launched or has failed, for per-rank callers that block until
+// their collective is complete (option "blocking").
+std::mutex g_mu;
+std::condition_variable g_round_cv;
+using Lock = std::unique_lock<std::mutex>;
 
 int fail(int code, const std::string& msg) {
     g_last_error = msg;
@@ -840,6 +852,7 @@ int drain_dispatch(mc_ep_world* w) {
         if (e) w->dispatch_rounds.front().state->failure = g_last_error;
         w->dispatch_rounds.pop_front();
         w->dispatch_base++;
+        g_round_cv.notify_all();
         if (e) return e;
     }
     return MC_EP_OK;
@@ -851,6 +864,7 @@ int drain_combine(mc_ep_world* w) {
         if (e) w->combine_rounds.front().state->failure = g_last_error;
         w->combine_rounds.pop_front();
         w->combine_base++;
+        g_round_cv.notify_all();
         if (e) return e;
     }
     return MC_EP_OK;
@@ -879,6 +893,22 @@ int round_not_ready(const Round* round) {
     return fail(MC_EP_ERR_PENDING,
                 "Failed: the call is a collective over the world's live ranks and not every one of them has "
                 "called it yet");
+}
+
+// Option "blocking": the caller is one of several threads, one per rank, each of which goes on to use its
+// results as soon as its call returns, as a process of the reference does.  The call therefore returns
+// only when the round has been launched (by the thread whose call completed it), so that whatever the
+// caller enqueues next on its stream is ordered behind the round.  Called with the lock held; the
+// wait gives it up.
+int wait_for_round(mc_ep_world* w, const std::shared_ptr<Round>& round, Lock& lock) {
+    if (w->tuning.blocking == 0) return MC_EP_OK;
+    const auto ready = [&] { return round->launched || !round->failure.empty(); };
+    const int ms = w->tuning.block_timeout_ms;
+    if (!g_round_cv.wait_for(lock, std::chrono::milliseconds(ms < 0 ? 0 : ms), ready))
+        return fail(MC_EP_ERR_PENDING, "Failed: the call waited " + std::to_string(ms) + " ms for the other live ranks "
+                                       "of its collective (option block_timeout_ms); it stays posted");
+    if (!round->failure.empty()) return round_not_ready(round.get());
+    return MC_EP_OK;
 }
 
 // The per-rank calls form a round out of several host calls, with events between streams: that
@@ -915,6 +945,7 @@ uint64_t mc_ep_get_buffer_size_hint(int max_tokens, int hidden, int num_ranks, i
 int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
     MC_ASSERT(out != nullptr);
     MC_ASSERT(num_ranks > 0 && num_ranks <= MC_EP_MAX_QP_COUNT);
+    Lock lock(g_mu);
     auto w = std::make_unique<mc_ep_world>();
     w->R = num_ranks;
     MC_HIP(hipGetDevice(&w->device));
@@ -945,6 +976,7 @@ int mc_ep_world_create(int num_ranks, mc_ep_world_t** out) {
 }
 
 int mc_ep_world_destroy(mc_ep_world_t* w) {
+    Lock lock(g_mu);
     delete w;   // ~mc_ep_world waits for the device and releases what the world owns
     return MC_EP_OK;
 }
@@ -953,6 +985,7 @@ int mc_ep_world_num_ranks(const mc_ep_world_t* w) { return w ? w->R : 0; }
 
 int mc_ep_world_set_rank_silent(mc_ep_world_t* w, int rank, int silent) {
     MC_ASSERT(w != nullptr && rank >= 0 && rank < w->R);
+    Lock lock(g_mu);
     const bool was_silent = w->silent[rank] != 0;
     w->silent[rank] = silent ? 1 : 0;
     if (was_silent && !silent) {
@@ -979,11 +1012,14 @@ static int* option_slot(Tuning& t, const char* name) {
     if (!strcmp(name, "routing_sum")) return &t.routing_sum;
     if (!strcmp(name, "combine_waves")) return &t.combine_waves;
     if (!strcmp(name, "combine_nt")) return &t.combine_nt;
+    if (!strcmp(name, "blocking")) return &t.blocking;
+    if (!strcmp(name, "block_timeout_ms")) return &t.block_timeout_ms;
     return nullptr;
 }
 
 int mc_ep_world_set_option(mc_ep_world_t* w, const char* name, int value) {
     MC_ASSERT(w != nullptr && name != nullptr);
+    Lock lock(g_mu);
     int* slot = option_slot(w->tuning, name);
     if (!slot) return fail(MC_EP_ERR_ASSERT, std::string("Failed: unknown option '") + name + "'");
     *slot = value;
@@ -992,6 +1028,7 @@ int mc_ep_world_set_option(mc_ep_world_t* w, const char* name, int value) {
 
 int mc_ep_world_get_option(const mc_ep_world_t* w, const char* name, int* value) {
     MC_ASSERT(w != nullptr && name != nullptr && value != nullptr);
+    Lock lock(g_mu);
     Tuning t = w->tuning;
     int* slot = option_slot(t, name);
     if (!slot) return fail(MC_EP_ERR_ASSERT, std::string("Failed: unknown option '") + name + "'");
@@ -1005,6 +1042,7 @@ int mc_ep_world_dispatch(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_
                          const uint64_t* recv_count_ptrs, const uint64_t* src_info_ptrs,
                          const uint64_t* layout_range_ptrs, int phases, uint64_t stream_ptr) {
     MC_ASSERT(w != nullptr);
+    Lock lock(g_mu);
     return world_dispatch_impl(w, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, max_tokens, num_experts,
                                use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
                                layout_range_ptrs, phases, (hipStream_t)stream_ptr);
@@ -1017,6 +1055,7 @@ int mc_ep_world_dispatch_noalloc(mc_ep_world_t* w, const uint64_t* x_ptrs, const
                                  const uint64_t* src_info_ptrs, const uint64_t* layout_range_ptrs,
                                  uint64_t stream_ptr) {
     MC_ASSERT(w != nullptr);
+    Lock lock(g_mu);
     return world_dispatch_impl(w, x_ptrs, topk_idx_ptrs, num_tokens, hidden, num_topk, max_tokens, num_experts,
                                use_fp8, recv_x_ptrs, recv_scales_ptrs, recv_count_ptrs, src_info_ptrs,
                                layout_range_ptrs, MC_EP_PHASE_ALL, (hipStream_t)stream_ptr, true);
@@ -1028,6 +1067,7 @@ int mc_ep_world_combine(mc_ep_world_t* w, const uint64_t* x_ptrs, const uint64_t
                         const int32_t* num_combined_tokens, int hidden, int num_topk, int max_tokens,
                         int num_experts, const uint64_t* combined_x_ptrs, int phases, uint64_t stream_ptr) {
     MC_ASSERT(w != nullptr);
+    Lock lock(g_mu);
     return world_combine_impl(w, x_ptrs, topk_idx_ptrs, topk_weights_ptrs, src_info_ptrs, layout_range_ptrs,
                               active_ranks_ptrs, num_combined_tokens, hidden, num_topk, max_tokens, num_experts,
                               combined_x_ptrs, phases, (hipStream_t)stream_ptr);
@@ -1040,6 +1080,7 @@ int mc_ep_world_combine_packed(mc_ep_world_t* w, const uint64_t* recv_x_ptrs, co
                                const int32_t* num_combined_tokens, int hidden, int num_topk, int max_tokens,
                                int num_experts, const uint64_t* combined_x_ptrs, int phases, uint64_t stream_ptr) {
     MC_ASSERT(w != nullptr);
+    Lock lock(g_mu);
     PackedSource ps;
     ps.packed = true;
     ps.scales = recv_scales_ptrs;
@@ -1053,6 +1094,7 @@ int mc_ep_world_cast_back(mc_ep_world_t* w, const uint64_t* recv_x_ptrs, const u
                           const uint64_t* recv_count_ptrs, uint64_t expert_factor_ptr, const uint64_t* out_ptrs,
                           int hidden, int num_topk, int max_tokens, int num_experts, uint64_t stream_ptr) {
     MC_ASSERT(w != nullptr);
+    Lock lock(g_mu);
     const int R = w->R;
     MC_ASSERT(num_experts > 0 && num_experts % R == 0);
     MC_ASSERT(hidden > 0 && hidden % 128 == 0);
@@ -1119,6 +1161,7 @@ int mc_ep_world_legacy_buffer_perf(mc_ep_world_t* w, const mc_ep_legacy_perf_ten
     const std::vector<int32_t> tokens((size_t)w->R, c->num_tokens);
 
     auto run_once = [&]() -> int {
+        Lock lock(g_mu);   // per step: the waits for the GPU below happen without it
         // the reference's cudaMemsetAsync(packed_recv_count) of every rank, in one launch
         MC_HIP(launch_clear_words(t->packed_recv_count_ptrs, w->R, c->num_local_experts, stream));
         int rc = world_dispatch_impl(w, t->x_ptrs, t->topk_idx_ptrs, tokens.data(), c->hidden, c->num_topk,
@@ -1178,6 +1221,7 @@ int mc_ep_world_legacy_buffer_perf(mc_ep_world_t* w, const mc_ep_legacy_perf_ten
 int mc_ep_buffer_create(mc_ep_world_t* w, int rank, int64_t num_ep_buffer_bytes, int disable_p2p,
                         mc_ep_buffer_t** out) {
     MC_ASSERT(w != nullptr && out != nullptr);
+    Lock lock(g_mu);
     MC_ASSERT(rank >= 0 && rank < w->R);
     MC_ASSERT(num_ep_buffer_bytes >= 0);
     auto* b = new mc_ep_buffer();
@@ -1190,12 +1234,14 @@ int mc_ep_buffer_create(mc_ep_world_t* w, int rank, int64_t num_ep_buffer_bytes,
 }
 
 int mc_ep_buffer_destroy(mc_ep_buffer_t* b) {
+    Lock lock(g_mu);
     delete b;
     return MC_EP_OK;
 }
 
 int mc_ep_buffer_pending_calls(const mc_ep_buffer_t* b, int* dispatch_pending, int* combine_pending) {
     MC_ASSERT(b != nullptr && dispatch_pending != nullptr && combine_pending != nullptr);
+    Lock lock(g_mu);
     const mc_ep_world* w = b->world;
     long long d = w->dispatch_calls[b->rank] - w->dispatch_base;
     long long c = w->combine_calls[b->rank] - w->combine_base;
@@ -1222,6 +1268,7 @@ int mc_ep_buffer_dispatch(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_p
     *event_out = nullptr;
     *hook_out = nullptr;
     if (int rc = refuse_capture(compute_stream_ptr)) return rc;
+    Lock lock(g_mu);
     mc_ep_world* w = b->world;
     const int num_ranks = w->R;
     // mooncake_ep_buffer.cpp:202-206
@@ -1261,6 +1308,7 @@ int mc_ep_buffer_dispatch(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_p
     std::shared_ptr<Round> state = pr.state;
 
     if (int e = drain_dispatch(w)) return e;
+    if (int e = wait_for_round(w, state, lock)) return e;
     if (async) {
         auto* ev = new mc_ep_event();
         ev->round = state;
@@ -1286,6 +1334,7 @@ int mc_ep_buffer_combine(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_pt
     *event_out = nullptr;
     *hook_out = nullptr;
     if (int rc = refuse_capture(compute_stream_ptr)) return rc;
+    Lock lock(g_mu);
     mc_ep_world* w = b->world;
     const int num_ranks = w->R;
     if (zero_copy)
@@ -1323,6 +1372,7 @@ int mc_ep_buffer_combine(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_pt
     std::shared_ptr<Round> state = pr.state;
 
     if (int e = drain_combine(w)) return e;
+    if (int e = wait_for_round(w, state, lock)) return e;
     if (async) {
         auto* ev = new mc_ep_event();
         ev->round = state;
@@ -1353,6 +1403,7 @@ int mc_ep_event_current_stream_wait(mc_ep_event_t* ev, uint64_t stream_ptr) {
         MC_HIP(hipStreamWaitEvent((hipStream_t)stream_ptr, ev->own, 0));
         return MC_EP_OK;
     }
+    Lock lock(g_mu);
     if (!ev->round || !ev->round->launched) return round_not_ready(ev->round.get());
     return ev->round->make_wait((hipStream_t)stream_ptr);
 }
@@ -1363,22 +1414,32 @@ int mc_ep_event_synchronize(mc_ep_event_t* ev) {
         MC_HIP(hipEventSynchronize(ev->own));
         return MC_EP_OK;
     }
-    if (!ev->round || !ev->round->launched) return round_not_ready(ev->round.get());
-    // an async caller's round always has its event; without one, the round's stream says the same
-    if (ev->round->done) MC_HIP(hipEventSynchronize(ev->round->done));
-    else MC_HIP(hipStreamSynchronize(ev->round->launch_stream));
+    hipEvent_t done = nullptr;
+    hipStream_t launch = nullptr;
+    {
+        Lock lock(g_mu);
+        if (!ev->round || !ev->round->launched) return round_not_ready(ev->round.get());
+        done = ev->round->done;
+        launch = ev->round->launch_stream;
+    }
+    // the wait itself happens without the lock; the handle keeps the round, and so its event, alive.
+    // An async caller's round always has its event; without one, the round's stream says the same.
+    if (done) MC_HIP(hipEventSynchronize(done));
+    else MC_HIP(hipStreamSynchronize(launch));
     return MC_EP_OK;
 }
 
 int mc_ep_event_destroy(mc_ep_event_t* ev) {
     if (!ev) return MC_EP_OK;
     if (ev->own) (void)hipEventDestroy(ev->own);
+    Lock lock(g_mu);   // the last handle of a round gives its event back to the pool
     delete ev;
     return MC_EP_OK;
 }
 
 int mc_ep_hook_call(mc_ep_hook_t* h) {
     MC_ASSERT(h != nullptr);
+    Lock lock(g_mu);
     if (!h->round || !h->round->launched) return round_not_ready(h->round.get());
     // the first hook of a round launched in two parts enqueues the second part (the reference's
     // RECV phase, mooncake_ep_buffer.cpp:330-335)
@@ -1389,6 +1450,7 @@ int mc_ep_hook_call(mc_ep_hook_t* h) {
 }
 
 int mc_ep_hook_destroy(mc_ep_hook_t* h) {
+    Lock lock(g_mu);
     delete h;
     return MC_EP_OK;
 }

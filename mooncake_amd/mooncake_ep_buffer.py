@@ -102,6 +102,12 @@ class Buffer:
         while len(posted) > pending:
             posted.popleft()
 
+    def _retain_if_posted(self, exc: RuntimeError, posted: collections.deque, tensors: tuple, kind: int) -> None:
+        """A blocking call that gave up waiting for its peers (option "blocking") has recorded its arguments all
+        the same: the round is enqueued when the peers arrive, so the tensors stay referenced as for any call."""
+        if "stays posted" in str(exc):
+            self._retain(posted, tensors, kind)
+
     @staticmethod
     def _hook_keeping(hook: Optional[Callable], tensors: tuple) -> Optional[Callable]:
         """The receive hook, holding the call's tensors until it has run: in hook mode nothing else
@@ -172,16 +178,20 @@ class Buffer:
             # column-major per expert: [L, H/128, R*max] storage viewed as [L, R*max, H/128]
             packed_recv_x_scales = torch.empty((num_local_experts, hidden // 128, rm), dtype=torch.float32,
                                                device=x.device).transpose(1, 2)
-        event, hook = self.runtime.dispatch(
-            x.data_ptr(), topk_idx.data_ptr(), active_ranks.data_ptr(), x.size(0), hidden, topk_idx.size(1),
-            num_max_dispatch_tokens_per_rank, num_experts, timeout_us, use_fp8, packed_recv_x.data_ptr(),
-            0 if packed_recv_x_scales is None else packed_recv_x_scales.data_ptr(), packed_recv_count.data_ptr(),
-            packed_recv_src_info.data_ptr(), packed_recv_layout_range.data_ptr(), async_finish, return_recv_hook,
-            _native_current_stream_ptr())
-        handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, hidden,
-                  num_experts)
         tensors_to_record = (x, topk_idx, active_ranks, packed_recv_x, packed_recv_x_scales, packed_recv_count,
                              packed_recv_src_info, packed_recv_layout_range)
+        try:
+            event, hook = self.runtime.dispatch(
+                x.data_ptr(), topk_idx.data_ptr(), active_ranks.data_ptr(), x.size(0), hidden, topk_idx.size(1),
+                num_max_dispatch_tokens_per_rank, num_experts, timeout_us, use_fp8, packed_recv_x.data_ptr(),
+                0 if packed_recv_x_scales is None else packed_recv_x_scales.data_ptr(), packed_recv_count.data_ptr(),
+                packed_recv_src_info.data_ptr(), packed_recv_layout_range.data_ptr(), async_finish, return_recv_hook,
+                _native_current_stream_ptr())
+        except RuntimeError as exc:
+            self._retain_if_posted(exc, self._posted_dispatch, tensors_to_record, 0)
+            raise
+        handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, hidden,
+                  num_experts)
         self._retain(self._posted_dispatch, tensors_to_record, 0)
         return ((packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x, packed_recv_count, handle,
                 EventOverlap(event, tensors_to_record if async_finish else None),
@@ -229,12 +239,16 @@ class Buffer:
             combined_x = out
         else:
             combined_x = torch.empty((topk_weights.size(0), hidden), dtype=x.dtype, device=x.device)
-        event, hook = self.runtime.combine(
-            x.data_ptr(), topk_idx.data_ptr(), topk_weights.data_ptr(), src_info.data_ptr(),
-            layout_range.data_ptr(), active_ranks.data_ptr(), x.size(0), topk_weights.size(0), hidden,
-            topk_weights.size(1), num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy,
-            combined_x.data_ptr(), async_finish, return_recv_hook, _native_current_stream_ptr())
         tensors_to_record = (x, topk_idx, topk_weights, active_ranks, src_info, layout_range, combined_x)
+        try:
+            event, hook = self.runtime.combine(
+                x.data_ptr(), topk_idx.data_ptr(), topk_weights.data_ptr(), src_info.data_ptr(),
+                layout_range.data_ptr(), active_ranks.data_ptr(), x.size(0), topk_weights.size(0), hidden,
+                topk_weights.size(1), num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy,
+                combined_x.data_ptr(), async_finish, return_recv_hook, _native_current_stream_ptr())
+        except RuntimeError as exc:
+            self._retain_if_posted(exc, self._posted_combine, tensors_to_record, 1)
+            raise
         self._retain(self._posted_combine, tensors_to_record, 1)
         return (combined_x, EventOverlap(event, tensors_to_record if async_finish else None),
                 self._hook_keeping(hook, tensors_to_record))

@@ -132,8 +132,9 @@ def test_ep_benchmark_zero_copy_is_refused_like_the_reference_build_without_it(g
 
 
 def test_native_driver_runs_without_python_in_the_loop(gpu_device):
-    """The C++ driver built from the C header alone: the per-rank Buffer calls in the three completion modes
-    (combined rows against the same multiply-add chain on the host, bit for bit), the whole-world self-check
+    """The C++ driver built from the C header alone: the per-rank Buffer calls in the three completion modes, from
+    one thread and from a thread per rank (combined rows against the same multiply-add chain on the host, bit for
+    bit), the whole-world self-check
     (per-expert row counts against a host count) and both timing loops."""
     import os
     import subprocess
@@ -148,6 +149,6 @@ def test_native_driver_runs_without_python_in_the_loop(gpu_device):
         run = subprocess.run([exe] + flags, capture_output=True, text=True, timeout=100)
         assert run.returncode == 0, run.stderr
         assert "us per step" in run.stdout and "native loop" in run.stdout
-        assert "combined rows equal the host chain" in run.stdout
+        assert "a thread per rank: combined rows equal the host chain" in run.stdout
     bad = subprocess.run([exe, "--ranks", "3", "--experts", "16"], capture_output=True, text=True, timeout=100)
     assert bad.returncode == 2 and "unusable shape" in bad.stderr

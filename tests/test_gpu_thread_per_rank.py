@@ -1,0 +1,145 @@
+"""A thread per rank, each running the reference's per-rank code unchanged: `Buffer(group, ...)`, `dispatch`,
+use the results at once, `combine`, use the result at once - what a process of the reference does
+(mooncake-ep/tests/test_ep_grid.py:60-119).  With the world's option "blocking" a per-rank call returns only
+when its collective has been launched, so whatever the thread does next with its outputs is ordered behind the
+kernels; every thread checks its own results against the oracle while the others are still running."""
+import threading
+import time
+
+import pytest
+import torch
+
+from mooncake_amd import Buffer, LogicalGroup
+from tests.gpu_util import announce
+from tests.test_gpu_buffer_lifetime import check_rank_dispatch, oracle_world, rank_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_threads(num_ranks, body):
+    """Runs body(rank) on one thread per rank; re-raises the first failure."""
+    errors = [None] * num_ranks
+
+    def guarded(r):
+        try:
+            body(r)
+        except BaseException as exc:       # noqa: BLE001 - reported to the main thread below
+            errors[r] = exc
+
+    threads = [threading.Thread(target=guarded, args=(r,), name=f"rank{r}") for r in range(num_ranks)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a rank's thread is still waiting"
+    for r, exc in enumerate(errors):
+        if exc is not None:
+            raise AssertionError(f"rank {r}: {exc!r}") from exc
+
+
+@pytest.mark.parametrize("mode", ["default", "async_finish", "return_recv_hook"])
+@pytest.mark.parametrize("use_fp8", [True, False], ids=["fp8", "bf16"])
+def test_thread_per_rank_uses_results_as_soon_as_the_call_returns(gpu_device, oracle, use_fp8, mode):
+    R, T, H, E, K, steps = 4, 48, 1024, 16, 4, 3
+    announce(f"thread per rank, fp8={use_fp8}, {mode}")
+    world, groups = LogicalGroup.make_world(R)
+    world.set_option("blocking", 1)
+    nbytes = Buffer.get_ep_buffer_size_hint(T, H, R, E)
+    inputs = [[rank_inputs(7000 + 10 * j + r, T - r, H, E, K) for r in range(R)] for j in range(steps)]
+    refs = [oracle_world(oracle, inputs[j], T, E, use_fp8) for j in range(steps)]
+    wants = []
+    for j in range(steps):
+        ref, xs, idxs, ws, nts = refs[j]
+        rows = oracle.cast_back(ref["recv_x"], ref["scales"] if use_fp8 else None, ref["recv_count"], None)
+        wants.append(oracle.combine(rows, idxs, ws, ref["src_info"], ref["layout_range"], nts, T, E))
+    kw = {"async_finish": mode == "async_finish", "return_recv_hook": mode == "return_recv_hook"}
+
+    def body(r):
+        torch.cuda.set_device(gpu_device)
+        buf = Buffer(groups[r], nbytes)
+        stream = torch.cuda.Stream()                       # every rank on a stream of its own
+        with torch.cuda.stream(stream):
+            for j in range(steps):
+                x, idx, w = (t.to(gpu_device, non_blocking=False) for t in inputs[j][r])
+                if r == j % R:
+                    time.sleep(0.02)                       # one rank is late: the others wait inside their calls
+                recv_x, recv_count, handle, event, hook = buf.dispatch(x, idx, None, T, E, -1, use_fp8=use_fp8, **kw)
+                if kw["async_finish"]:
+                    event.current_stream_wait()
+                if kw["return_recv_hook"]:
+                    hook()
+                # used at once, on this thread's stream, while other ranks may still be inside their calls
+                check_rank_dispatch(refs[j][0], r, recv_x, recv_count, handle, use_fp8)
+                if use_fp8:
+                    payload, scales = recv_x
+                    g = scales.size(-1)
+                    expert_out = (payload.float().view(*payload.shape[:2], g, 128) * scales.unsqueeze(-1)) \
+                        .view(payload.shape).to(torch.bfloat16)
+                else:
+                    expert_out = recv_x
+                out, event, hook = buf.combine(expert_out, idx, w, None, -1, handle, **kw)
+                if kw["async_finish"]:
+                    event.current_stream_wait()
+                if kw["return_recv_hook"]:
+                    hook()
+                n = x.size(0)
+                assert torch.equal(out.cpu().view(torch.int16), wants[j][r, :n].view(torch.int16)), f"step {j}"
+
+    _run_threads(R, body)
+
+
+def test_a_blocked_call_gives_up_after_the_timeout_and_stays_posted(gpu_device, oracle):
+    R, T, H, E, K = 2, 32, 512, 8, 2
+    announce("blocking call times out, the round completes later")
+    world, groups = LogicalGroup.make_world(R)
+    world.set_option("blocking", 1)
+    world.set_option("block_timeout_ms", 150)
+    nbytes = Buffer.get_ep_buffer_size_hint(T, H, R, E)
+    bufs = [Buffer(g, nbytes) for g in groups]
+    per_rank = [rank_inputs(7100 + r, T, H, E, K) for r in range(R)]
+    dev = [tuple(t.to(gpu_device) for t in per_rank[r]) for r in range(R)]
+    outs = [dict(recv_x=torch.empty((E // R, R * T, H), dtype=torch.bfloat16, device=gpu_device),
+                 recv_count=torch.empty((E // R,), dtype=torch.int32, device=gpu_device),
+                 src_info=torch.empty((E // R, R * T), dtype=torch.int32, device=gpu_device),
+                 layout_range=torch.empty((E // R, R), dtype=torch.int64, device=gpu_device)) for _ in range(R)]
+    active = torch.ones(R, dtype=torch.int32, device=gpu_device)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def post(r):
+        x, idx, _ = dev[r]
+        o = outs[r]
+        return bufs[r].runtime.dispatch(x.data_ptr(), idx.data_ptr(), active.data_ptr(), T, H, K, T, E, -1, False,
+                                        o["recv_x"].data_ptr(), 0, o["recv_count"].data_ptr(),
+                                        o["src_info"].data_ptr(), o["layout_range"].data_ptr(), False, False, stream)
+
+    t0 = time.perf_counter()
+    with pytest.raises(RuntimeError, match="waited 150 ms"):
+        post(0)                                            # nobody else is calling
+    assert 0.1 < time.perf_counter() - t0 < 5.0
+    assert bufs[0].runtime.pending_calls() == (1, 0)      # the call stays posted
+    post(1)                                                # completes the round and returns at once
+    torch.cuda.synchronize()
+    assert bufs[0].runtime.pending_calls() == (0, 0)
+    ref, *_ = oracle_world(oracle, per_rank, T, E, False)
+    for r in range(R):
+        o = outs[r]
+        check_rank_dispatch(ref, r, o["recv_x"], o["recv_count"], (o["src_info"], o["layout_range"]), False)
+
+
+def test_without_the_option_one_thread_still_drives_all_ranks(gpu_device, oracle):
+    """The default stays what it was: calls return at once, and the last rank's call launches the round."""
+    R, T, H, E, K = 2, 32, 512, 8, 2
+    announce("non-blocking default")
+    world, groups = LogicalGroup.make_world(R)
+    assert world.get_option("blocking") == 0
+    nbytes = Buffer.get_ep_buffer_size_hint(T, H, R, E)
+    bufs = [Buffer(g, nbytes) for g in groups]
+    per_rank = [rank_inputs(7200 + r, T, H, E, K) for r in range(R)]
+    t0 = time.perf_counter()
+    res = [bufs[r].dispatch(per_rank[r][0].to(gpu_device), per_rank[r][1].to(gpu_device), None, T, E, -1, use_fp8=False)
+           for r in range(R)]
+    assert time.perf_counter() - t0 < 5.0
+    torch.cuda.synchronize()
+    ref, *_ = oracle_world(oracle, per_rank, T, E, False)
+    for r in range(R):
+        check_rank_dispatch(ref, r, res[r][0], res[r][1], res[r][2], False)
