@@ -15,7 +15,8 @@
  *
  * Threads: the library's host bookkeeping sits behind one process-wide lock,
  * so any thread may call any function; a call holds the lock while it records
- * arguments and enqueues kernels, never while it waits for the GPU.  What the
+ * arguments and enqueues kernels, not while it waits for a collective's peers
+ * or results.  What the
  * lock cannot give is order: calls of one rank must come from one thread at a
  * time (the reference's buffer is not thread-safe either,
  * mooncake_ep_buffer.cpp:215-218), and with one driver thread for all ranks a

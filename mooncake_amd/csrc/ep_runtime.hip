@@ -41,7 +41,8 @@ thread_local std::string g_last_error;
 
 // One lock for the host bookkeeping of every world, buffer, round, event and hook of the process (an
 // EventHandle may outlive its world, so the lock cannot live in the world): entry points take it for as
-// long as they touch that state and enqueue work, never while they wait for the GPU.  g_round_cv is
+// long as they touch that state and enqueue work, not while they wait for a collective's peers or for
+// its results (the short waits of set-up - a world's destruction, scratch that grows - are inside).  g_round_cv is
 // signalled whenever a round has been launched or has failed, for per-rank callers that block until
 // their collective is complete (option "blocking").
 std::mutex g_mu;
