@@ -5,6 +5,6 @@
 `libmooncake_ep_hip.so` and fail loudly without it.
 """
 from . import ep  # noqa: F401
-from .mooncake_ep_buffer import Buffer, EventOverlap, LogicalGroup  # noqa: F401
+from .mooncake_ep_buffer import Buffer, EventOverlap, LogicalGroup, spawn_ranks  # noqa: F401
 
-__all__ = ["ep", "Buffer", "EventOverlap", "LogicalGroup"]
+__all__ = ["ep", "Buffer", "EventOverlap", "LogicalGroup", "spawn_ranks"]

@@ -57,6 +57,50 @@ class LogicalGroup:
         return world, [LogicalGroup(world, r) for r in range(num_ranks)]
 
 
+def spawn_ranks(fn: Callable, num_ranks: int, args: tuple = (), join_timeout: Optional[float] = None,
+                block_timeout_ms: Optional[int] = None) -> list:
+    """Runs `fn(rank, group, *args)` on one thread per logical rank of a fresh world and returns the ranks'
+    results: the counterpart, for logical ranks, of the `torch.multiprocessing.spawn(worker, nprocs=world_size)`
+    that the reference's tests start their per-rank code with (mooncake-ep/tests/test_ep_grid.py:412-430).
+    `group` stands in for the process group (`Buffer(group, ...)`).  The world's per-rank calls block until their
+    collective has been enqueued (option "blocking"), so `fn` may use a call's results as soon as the call
+    returns, as a process of the reference does.  The first exception of any rank is raised again here."""
+    import threading
+    world, groups = LogicalGroup.make_world(num_ranks)
+    world.set_option("blocking", 1)
+    if block_timeout_ms is not None:
+        world.set_option("block_timeout_ms", int(block_timeout_ms))
+    device = torch.cuda.current_device() if torch.cuda.is_available() else None
+    results: list = [None] * num_ranks
+    errors: list = [None] * num_ranks
+
+    def run(rank: int) -> None:
+        try:
+            if device is not None:
+                torch.cuda.set_device(device)       # the current device is per thread
+            results[rank] = fn(rank, groups[rank], *args)
+        except BaseException as exc:                # noqa: BLE001 - handed to the caller below
+            errors[rank] = exc
+            # a rank that stops calling would leave its peers waiting for the time limit: take it out of their rounds
+            try:
+                world.set_rank_silent(rank)
+            except Exception:                       # noqa: BLE001
+                pass
+
+    threads = [threading.Thread(target=run, args=(r,), name=f"ep-rank-{r}") for r in range(num_ranks)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(join_timeout)
+    alive = [t.name for t in threads if t.is_alive()]
+    for rank, exc in enumerate(errors):
+        if exc is not None:
+            raise RuntimeError(f"logical rank {rank} failed: {exc!r}") from exc
+    if alive:
+        raise TimeoutError(f"ranks still running after {join_timeout} s: {alive}")
+    return results
+
+
 class EventOverlap:
     """Event wrapper with the `with` protocol (reference :34-89)."""
 

@@ -3,38 +3,16 @@ use the results at once, `combine`, use the result at once - what a process of t
 (mooncake-ep/tests/test_ep_grid.py:60-119).  With the world's option "blocking" a per-rank call returns only
 when its collective has been launched, so whatever the thread does next with its outputs is ordered behind the
 kernels; every thread checks its own results against the oracle while the others are still running."""
-import threading
 import time
 
 import pytest
 import torch
 
-from mooncake_amd import Buffer, LogicalGroup
+from mooncake_amd import Buffer, LogicalGroup, spawn_ranks
 from tests.gpu_util import announce
 from tests.test_gpu_buffer_lifetime import check_rank_dispatch, oracle_world, rank_inputs
 
 pytestmark = pytest.mark.gpu
-
-
-def _run_threads(num_ranks, body):
-    """Runs body(rank) on one thread per rank; re-raises the first failure."""
-    errors = [None] * num_ranks
-
-    def guarded(r):
-        try:
-            body(r)
-        except BaseException as exc:       # noqa: BLE001 - reported to the main thread below
-            errors[r] = exc
-
-    threads = [threading.Thread(target=guarded, args=(r,), name=f"rank{r}") for r in range(num_ranks)]
-    for t in threads:
-        t.start()
-    for t in threads:
-        t.join(timeout=100)
-    assert not any(t.is_alive() for t in threads), "a rank's thread is still waiting"
-    for r, exc in enumerate(errors):
-        if exc is not None:
-            raise AssertionError(f"rank {r}: {exc!r}") from exc
 
 
 @pytest.mark.parametrize("mode", ["default", "async_finish", "return_recv_hook"])
@@ -42,8 +20,6 @@ def _run_threads(num_ranks, body):
 def test_thread_per_rank_uses_results_as_soon_as_the_call_returns(gpu_device, oracle, use_fp8, mode):
     R, T, H, E, K, steps = 4, 48, 1024, 16, 4, 3
     announce(f"thread per rank, fp8={use_fp8}, {mode}")
-    world, groups = LogicalGroup.make_world(R)
-    world.set_option("blocking", 1)
     nbytes = Buffer.get_ep_buffer_size_hint(T, H, R, E)
     inputs = [[rank_inputs(7000 + 10 * j + r, T - r, H, E, K) for r in range(R)] for j in range(steps)]
     refs = [oracle_world(oracle, inputs[j], T, E, use_fp8) for j in range(steps)]
@@ -54,9 +30,9 @@ def test_thread_per_rank_uses_results_as_soon_as_the_call_returns(gpu_device, or
         wants.append(oracle.combine(rows, idxs, ws, ref["src_info"], ref["layout_range"], nts, T, E))
     kw = {"async_finish": mode == "async_finish", "return_recv_hook": mode == "return_recv_hook"}
 
-    def body(r):
-        torch.cuda.set_device(gpu_device)
-        buf = Buffer(groups[r], nbytes)
+    def worker(r, group):
+        assert group.rank() == r and group.size() == R
+        buf = Buffer(group, nbytes)
         stream = torch.cuda.Stream()                       # every rank on a stream of its own
         with torch.cuda.stream(stream):
             for j in range(steps):
@@ -84,8 +60,29 @@ def test_thread_per_rank_uses_results_as_soon_as_the_call_returns(gpu_device, or
                     hook()
                 n = x.size(0)
                 assert torch.equal(out.cpu().view(torch.int16), wants[j][r, :n].view(torch.int16)), f"step {j}"
+        return r * 10
 
-    _run_threads(R, body)
+    assert spawn_ranks(worker, R, join_timeout=100) == [0, 10, 20, 30]
+
+
+def test_a_rank_that_fails_is_reported_and_its_peers_are_not_left_waiting(gpu_device):
+    R, T, H, E, K = 3, 16, 256, 6, 2
+    announce("spawn_ranks: one rank raises")
+    nbytes = Buffer.get_ep_buffer_size_hint(T, H, R, E)
+
+    def worker(r, group):
+        buf = Buffer(group, nbytes)
+        if r == 1:
+            raise ValueError("rank 1 gives up")
+        x, idx, _ = (t.to(gpu_device) for t in rank_inputs(7300 + r, T, H, E, K))
+        _, recv_count, _, _, _ = buf.dispatch(x, idx, None, T, E, -1, use_fp8=False)
+        return int(recv_count.sum())
+
+    t0 = time.perf_counter()
+    with pytest.raises(RuntimeError, match="logical rank 1 failed.*rank 1 gives up"):
+        spawn_ranks(worker, R, join_timeout=60, block_timeout_ms=20000)
+    # the failed rank was taken out of the collective: the others did not sit out the time limit
+    assert time.perf_counter() - t0 < 15.0
 
 
 def test_a_blocked_call_gives_up_after_the_timeout_and_stays_posted(gpu_device, oracle):
