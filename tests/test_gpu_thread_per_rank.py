@@ -140,3 +140,53 @@ def test_without_the_option_one_thread_still_drives_all_ranks(gpu_device, oracle
     ref, *_ = oracle_world(oracle, per_rank, T, E, False)
     for r in range(R):
         check_rank_dispatch(ref, r, res[r][0], res[r][1], res[r][2], False)
+
+
+@pytest.mark.parametrize("use_fp8", [False, True], ids=["bf16", "fp8"])
+@pytest.mark.parametrize("mode", ["default", "async_finish", "return_recv_hook"])
+def test_reference_grid_worker_on_threads_with_a_rank_that_dies(gpu_device, use_fp8, mode):
+    """The reference's per-rank worker (mooncake-ep/tests/test_ep_grid.py:60-119, :160-173): dispatch, mock expert,
+    combine, closed form; two steps, and rank 1 stops calling after the first (the reference's os._exit(0),
+    :121-158, forced here from the host), so the survivors' second step runs without it."""
+    from tests.test_gpu_buffer_api import dequantize_fp8, grid_inputs
+    R, max_tokens, hidden, num_experts, top_k, fail_rank = 4, 64, 1024, 32, 4, 1
+    announce(f"grid worker on threads, fp8={use_fp8}, {mode}")
+    L = num_experts // R
+    nbytes = Buffer.get_ep_buffer_size_hint(max_tokens, hidden, R, num_experts)
+    kw = {"async_finish": mode == "async_finish", "return_recv_hook": mode == "return_recv_hook"}
+
+    def worker(rank, group):
+        buf = Buffer(group, nbytes)
+        x, idx, w = grid_inputs(rank, R, max_tokens, hidden, num_experts, top_k, gpu_device)
+        active = torch.ones(R, dtype=torch.int32, device=gpu_device)
+        for step in range(2):
+            if step == 1 and rank == fail_rank:
+                group.world.set_rank_silent(rank)          # this rank's process is gone
+                return "dead"
+            timeout_us = 5000 if step == 1 else -1
+            recv_x, recv_count, handle, event, hook = buf.dispatch(x, idx, active, max_tokens, num_experts, timeout_us,
+                                                                   use_fp8=use_fp8, **kw)
+            if kw["return_recv_hook"]:
+                hook()
+            if kw["async_finish"]:
+                event.current_stream_wait()
+            recv_bf16 = dequantize_fp8(*recv_x) if use_fp8 else recv_x
+            factor = (torch.arange(rank * L, (rank + 1) * L, device=gpu_device).float() * 0.1 + 1.0).view(L, 1, 1)
+            expert_out = (recv_bf16.float() * factor).to(torch.bfloat16).contiguous()
+            out, event, hook = buf.combine(expert_out, idx, w, active, timeout_us, handle, out=torch.zeros_like(x), **kw)
+            if kw["return_recv_hook"]:
+                hook()
+            if kw["async_finish"]:
+                event.current_stream_wait()
+            factors = idx.float() * 0.1 + 1.0
+            if step == 1:
+                assert active[fail_rank].item() == 0 and active.sum().item() == R - 1
+                factors = factors * (idx // L != fail_rank).float()
+            else:
+                assert active.sum().item() == R
+            expected = (x.float() * (factors * w).sum(dim=1, keepdim=True)).to(torch.bfloat16)
+            assert not torch.isnan(out.float()).any()
+            torch.testing.assert_close(out, expected, rtol=0.15 if use_fp8 else 5e-2, atol=5e-3 if use_fp8 else 1e-3)
+        return "alive"
+
+    assert spawn_ranks(worker, R, join_timeout=100) == ["alive", "dead", "alive", "alive"]
