@@ -3,8 +3,10 @@
 Same three modes, signatures, defaults and error conditions as the reference's
 mooncake-ep/benchmarks/ep_benchmark/routing.py (uniform :19-44, k-hot :47-103,
 Zipf :106-146, table :149-153).  Each generator draws from one seeded
-`torch.Generator` in the order the reference does (scores, then weights), so a
-seed names the same workload on the same device type.
+`torch.Generator` in the order the reference's text does (scores, then
+weights).  The tests check the definitions (distinct experts, expected loads,
+error conditions); that a seed reproduces the reference's tensors value for
+value is not tested, because the reference is not run here.
 """
 from __future__ import annotations
 
