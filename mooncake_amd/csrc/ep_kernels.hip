@@ -851,8 +851,12 @@ __device__ __forceinline__ uint32_t scale_round_twice(float a, float b, float s,
 // and row; a 128-element scale group is 8 lanes, and the scales of a row sit R*max floats apart in the
 // column-major layout), 512 elements of a bf16 payload.  Lanes 0..K-1 find the K rows as reduce_kernel
 // does; a masked, inactive or unknown selection reads the zero row with weight 0.
+//
+// Up to top-8 the register budget is that of eight waves per SIMD: left to itself the compiler spends
+// twice as many on the variant without a factor (to hoist every load), and at four waves per SIMD that
+// variant ran 5 % slower.  (Sixteen rows in flight do not fit that budget.)
 template <int KMAX, bool FP8, bool FACTOR, bool DIRECT>
-__global__ __launch_bounds__(512) void reduce_packed_kernel(const uint64_t* __restrict__ tbl,
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ? 8 : 4, 8))) void reduce_packed_kernel(const uint64_t* __restrict__ tbl,
                                                              const CombineRoute* __restrict__ routes, uint32_t stamp,
                                                              RoutingScratch sc, CombineSource cs,
                                                              const void* __restrict__ zero_row,
