@@ -14,6 +14,7 @@
 #include <pybind11/pybind11.h>
 #include <pybind11/stl.h>
 
+#include <atomic>
 #include <cstdint>
 #include <functional>
 #include <map>
@@ -49,7 +50,7 @@ using I32s = std::vector<int32_t>;
 struct World {
     mc_ep_world_t* h = nullptr;
     int num_ranks = 0;
-    bool blocking = false;   // option "blocking": per-rank calls wait for their peers, so they must not hold the GIL
+    std::atomic<bool> blocking{false};   // option "blocking": per-rank calls wait for their peers, so they must not hold the GIL
     explicit World(int n) : num_ranks(n) { check(mc_ep_world_create(n, &h)); }
     World(const World&) = delete;
     World& operator=(const World&) = delete;
