@@ -17,9 +17,11 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("mode", ["default", "async_finish", "return_recv_hook"])
 @pytest.mark.parametrize("use_fp8", [True, False], ids=["fp8", "bf16"])
-def test_thread_per_rank_uses_results_as_soon_as_the_call_returns(gpu_device, oracle, use_fp8, mode):
+@pytest.mark.parametrize("own_stream", [True, False], ids=["own_streams", "shared_stream"])
+def test_thread_per_rank_uses_results_as_soon_as_the_call_returns(gpu_device, oracle, use_fp8, mode, own_stream):
     R, T, H, E, K, steps = 4, 48, 1024, 16, 4, 3
-    announce(f"thread per rank, fp8={use_fp8}, {mode}")
+    announce(f"thread per rank, fp8={use_fp8}, {mode}, own_stream={own_stream}")
+    shared = torch.cuda.Stream()
     nbytes = Buffer.get_ep_buffer_size_hint(T, H, R, E)
     inputs = [[rank_inputs(7000 + 10 * j + r, T - r, H, E, K) for r in range(R)] for j in range(steps)]
     refs = [oracle_world(oracle, inputs[j], T, E, use_fp8) for j in range(steps)]
@@ -33,7 +35,9 @@ def test_thread_per_rank_uses_results_as_soon_as_the_call_returns(gpu_device, or
     def worker(r, group):
         assert group.rank() == r and group.size() == R
         buf = Buffer(group, nbytes)
-        stream = torch.cuda.Stream()                       # every rank on a stream of its own
+        # every rank on a stream of its own (rounds then run on the world's stream, fenced against each), or
+        # all on one stream (rounds run there)
+        stream = torch.cuda.Stream() if own_stream else shared
         with torch.cuda.stream(stream):
             for j in range(steps):
                 x, idx, w = (t.to(gpu_device, non_blocking=False) for t in inputs[j][r])
