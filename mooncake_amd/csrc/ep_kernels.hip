@@ -832,10 +832,16 @@ __device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf2));   // v_cvt_pk_bf16_f32
 }
 
+// x rounded to bf16 (nearest even) and kept as an f32: the conversion of the pair (0, x) leaves bf16(x) in
+// the upper half of the register, which is that value's f32 encoding - one instruction where packing two
+// values and unpacking them again takes three for two
+__device__ __forceinline__ float round_bf16(float x) {
+    return __uint_as_float(pack_bf16_rne(0.0f, x));
+}
+
 // out = bf16(bf16(a * s) * f), both roundings to nearest even, for a pair
 __device__ __forceinline__ uint32_t scale_round_twice(float a, float b, float s, float f) {
-    const uint32_t once = pack_bf16_rne(a * s, b * s);
-    return pack_bf16_rne(bf16_lo(once) * f, bf16_hi(once) * f);
+    return pack_bf16_rne(round_bf16(a * s) * f, round_bf16(b * s) * f);
 }
 
 // Combine straight from the packed layout dispatch wrote: what cast_back_kernel followed by
@@ -971,21 +977,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
                 typedef float f2 __attribute__((ext_vector_type(2)));
                 const f2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)u[j], false);
                 const f2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)u[j], true);
-                uint32_t lo = pack_bf16_rne(a.x * sv[k], a.y * sv[k]);
-                uint32_t hi = pack_bf16_rne(b.x * sv[k], b.y * sv[k]);
-                if (FACTOR) {
-                    lo = pack_bf16_rne(bf16_lo(lo) * fk[k], bf16_hi(lo) * fk[k]);
-                    hi = pack_bf16_rne(bf16_lo(hi) * fk[k], bf16_hi(hi) * fk[k]);
+                float e[4] = {round_bf16(a.x * sv[k]), round_bf16(a.y * sv[k]), round_bf16(b.x * sv[k]),
+                              round_bf16(b.y * sv[k])};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (FACTOR) e[i] = round_bf16(e[i] * fk[k]);
+                    acc[4 * j + i] = __builtin_fmaf(e[i], wk[k], acc[4 * j + i]);
                 }
-                acc[4 * j + 0] = __builtin_fmaf(bf16_lo(lo), wk[k], acc[4 * j + 0]);
-                acc[4 * j + 1] = __builtin_fmaf(bf16_hi(lo), wk[k], acc[4 * j + 1]);
-                acc[4 * j + 2] = __builtin_fmaf(bf16_lo(hi), wk[k], acc[4 * j + 2]);
-                acc[4 * j + 3] = __builtin_fmaf(bf16_hi(hi), wk[k], acc[4 * j + 3]);
             } else {
-                uint32_t x = u[j];
-                if (FACTOR) x = pack_bf16_rne(bf16_lo(x) * fk[k], bf16_hi(x) * fk[k]);
-                acc[2 * j + 0] = __builtin_fmaf(bf16_lo(x), wk[k], acc[2 * j + 0]);
-                acc[2 * j + 1] = __builtin_fmaf(bf16_hi(x), wk[k], acc[2 * j + 1]);
+                float e[2] = {bf16_lo(u[j]), bf16_hi(u[j])};
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    if (FACTOR) e[i] = round_bf16(e[i] * fk[k]);
+                    acc[2 * j + i] = __builtin_fmaf(e[i], wk[k], acc[2 * j + i]);
+                }
             }
         }
     }
