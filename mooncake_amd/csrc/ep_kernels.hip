@@ -680,7 +680,8 @@ __global__ __launch_bounds__(256) void resolve_kernel(const uint64_t* __restrict
 }
 
 // Where combine finds the row of selection `lane` of token (r, t) when the handle is the last
-// dispatch's: the pack kernel left expert * R*max + row in selrow (-1: the selection went nowhere).
+// dispatch's: the pack kernel left expert * R*max + row in selrow (-1: the selection went nowhere);
+// the row counts only while topk_idx still names that expert.
 // One load away from the payload when the ranks' row tensors are evenly spaced (the address then comes
 // from kernel arguments), two otherwise (rank table).  `live` is loaded but not waited for: whether
 // the owner is active only decides the weight, so the caller issues its payload loads first.
@@ -693,14 +694,19 @@ struct DirectRow {
 };
 
 __device__ __forceinline__ DirectRow direct_row(const uint64_t* __restrict__ tbl, const RoutingScratch& sc,
-                                                const RankPtr& x, int R, int E, int K, int max_tokens, int r, int t,
-                                                int lane) {
+                                                const RankPtr& x, const RankPtr& topk_idx, int R, int E, int K,
+                                                int max_tokens, int r, int t, int lane) {
     const int RM = R * max_tokens;
     const int L = E / R;
     const uint64_t active = tbl[CF_ACTIVE * R + r];
-    const int sr = sc.selrow[((int64_t)r * max_tokens + t) * K + (lane < K ? lane : 0)];
+    const int li = lane < K ? lane : 0;
+    // The selection as combine is given it, next to the row the dispatch left (two independent loads):
+    // combine reads topk_idx itself and skips what is negative there (mooncake_ep_kernel.cu:719-732), so
+    // a selection masked - or pointed elsewhere - after the dispatch has no row.
+    const int64_t now = ((const MCEP_GLOBAL int64_t*)(uintptr_t)rank_ptr(tbl, topk_idx, CF_TOPK_IDX, R, r))[(int64_t)t * K + li];
+    const int sr = sc.selrow[((int64_t)r * max_tokens + t) * K + li];
     DirectRow d;
-    d.has = lane < K && sr >= 0;
+    d.has = lane < K && sr >= 0 && now == (int64_t)(sr / RM);
     d.e = d.has ? sr / RM : 0;
     d.slot = d.has ? sr - d.e * RM : 0;
     d.q = d.e / L;
@@ -746,7 +752,7 @@ __global__ __launch_bounds__(512) void reduce_kernel(const uint64_t* __restrict_
         if (t >= T) return;
         const uint64_t w_row = rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (uint64_t)((int64_t)t * K) * 4;
         const float wl = load_f32(w_row + (uint64_t)(lane < K ? lane : 0) * 4);
-        const DirectRow d = direct_row(tbl, sc, cs.x, R, E, K, max_tokens, r, t, lane);
+        const DirectRow d = direct_row(tbl, sc, cs.x, cs.topk_idx, R, E, K, max_tokens, r, t, lane);
         if (d.has && d.base != 0) {
             src = d.base + (uint64_t)d.grow * (uint64_t)H * 2;
             w = wl;
@@ -902,7 +908,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
         if (DIRECT) {
             const uint64_t w_row = rank_ptr(tbl, cs.topk_weights, CF_TOPK_W, R, r) + (uint64_t)((int64_t)t * K) * 4;
             wl = load_f32(w_row + (uint64_t)(lane < K ? lane : 0) * 4);
-            const DirectRow d = direct_row(tbl, sc, cs.x, R, E, K, max_tokens, r, t, lane);
+            const DirectRow d = direct_row(tbl, sc, cs.x, cs.topk_idx, R, E, K, max_tokens, r, t, lane);
             ok = d.has;
             e = d.e;
             slot = d.slot;

@@ -413,7 +413,10 @@ int finish_round(mc_ep_world* w, Round* round) {
     if (!round->finish) return MC_EP_OK;
     const std::function<int()> rest = std::move(round->finish);
     round->finish = nullptr;
-    if (w->unfinished.get() == round) w->unfinished.reset();
+    // the world's reference may be the last one (every hook of the round dropped without being called):
+    // it is held here until the second part has been enqueued and its outcome recorded in the round
+    std::shared_ptr<Round> keep;
+    if (w->unfinished.get() == round) keep = std::move(w->unfinished);
     const int e = rest();
     if (e) round->failure = g_last_error;
     return e;
@@ -620,10 +623,10 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
 
     // Is this the handle (and the routing input) of the last dispatch?  Then the
-    // packed row of every selection is already known on the device.  Like the
-    // reference, this relies on topk_idx being unchanged between a dispatch and
-    // the combine of its handle (mooncake_ep_kernel.cu:734 finds a token's rows
-    // by its dispatch-time expert indices).
+    // packed row of every selection is already known on the device.  The kernel
+    // still reads topk_idx as combine is given it, as the reference's does
+    // (mooncake_ep_kernel.cu:719-732): a selection that no longer names the
+    // expert it was dispatched to (masked to -1 in place, say) contributes nothing.
     const auto& ld = w->last;
     bool direct = w->tuning.combine_direct != 0 && ld.valid && ld.data_done && ld.hidden == hidden &&
                   (long long)num_experts * R * max_tokens < 0x7fffffffll && ld.num_topk == num_topk &&

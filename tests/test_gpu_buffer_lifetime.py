@@ -309,6 +309,30 @@ def test_next_dispatch_enqueues_a_second_part_nobody_asked_for(gpu_device, oracl
             check_rank_dispatch(ref, r, outs[r][0], outs[r][1], outs[r][2], True)
 
 
+def test_next_dispatch_after_every_hook_was_dropped(gpu_device, oracle):
+    """The hooks of a two-part round are the only other owners of its state once the round has left the
+    queue.  Dropped without being called, they leave the world's own reference as the last one - and the
+    next dispatch, which has to enqueue the second part itself, must keep the round alive while it does."""
+    R, T, H, E, K = 2, 32, 1024, 8, 2
+    announce("return_recv_hook: hooks destroyed uncalled, then a second dispatch")
+    world, bufs = make_world(R, T, H, E)
+    a = [rank_inputs(410 + r, T, H, E, K) for r in range(R)]
+    b = [rank_inputs(510 + r, T, H, E, K) for r in range(R)]
+    outs_a = [bufs[r].dispatch(a[r][0].cuda(), a[r][1].cuda(), None, T, E, -1, use_fp8=True, return_recv_hook=True)
+              for r in range(R)]
+    assert bufs[0].runtime.pending_calls() == (1, 0)
+    kept_a = [o[:3] for o in outs_a]
+    del outs_a                                   # the hook closures go, and the library's hook objects with them
+    gc.collect()
+    outs_b = [bufs[r].dispatch(b[r][0].cuda(), b[r][1].cuda(), None, T, E, -1, use_fp8=True) for r in range(R)]
+    torch.cuda.synchronize()
+    assert bufs[0].runtime.pending_calls() == (0, 0)
+    for ins, outs in ((a, kept_a), (b, outs_b)):
+        ref, *_ = oracle_world(oracle, ins, T, E, True)
+        for r in range(R):
+            check_rank_dispatch(ref, r, outs[r][0], outs[r][1], outs[r][2], True)
+
+
 def test_silent_rank_comes_back(gpu_device, oracle):
     R, T, H, E, K = 3, 32, 512, 12, 3
     announce("a silent rank rejoins the world")
