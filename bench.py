@@ -53,6 +53,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-flushed", action="store_true", help="skip the cache-flushed timing")
     ap.add_argument("--no-buffer-api", action="store_true", help="skip the per-rank Buffer API timing")
+    ap.add_argument("--no-small-world", action="store_true", help="skip the launch-bound small-world shapes")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget for the cpu_baseline sample")
     ap.add_argument("--kernel-iters", type=int, default=30, help="timed launches per kernel for the roofline figures")
     ap.add_argument("--opt", action="append", default=[], help="library tuning option, name=value")
@@ -268,6 +269,56 @@ def time_python_buffer(h, steps, warmup):
         step()
     torch.cuda.synchronize()
     return {"us_per_step": round((time.perf_counter() - t0) / n * 1e6, 2), "steps": n}
+
+
+def time_small_world(iters):
+    """Launch-bound shapes, reported beside the headline and never part of `value`: the world one deployed
+    rank of the DeepSeek-V3 decode configuration sees by itself (1 x 128 tokens, hidden 7168, 256 experts,
+    top-8, fp8: 9.4 MB / 16.5 MB of algorithmic traffic, 1.2 / 2.1 us at the HBM peak) and the contract's
+    CPU-reference case (4 x 128 tokens, hidden 2048, 16 experts, top-4, bf16).  Each with the one-launch
+    dispatch of small worlds on and off: device time per call with calls issued back to back (dispatches in a
+    row, combines in a row, whole steps in a row) and the kernel launches one call makes."""
+    import torch
+    from mooncake_amd.harness import WorldHarness
+    from mooncake_amd.workloads import CONFIGS, EPConfig, algorithmic_bytes, generate
+    shapes = {"one_rank_dsv3_decode": EPConfig("one_rank_dsv3_decode", 1, 128, 7168, 256, 8, True),
+              "cpu_check": CONFIGS["cpu_check"]}
+    out = {}
+    for name, cfg in shapes.items():
+        data = generate(cfg, seed=0)
+        S = int((data["topk_idx"] >= 0).sum())
+        alg = algorithmic_bytes(cfg, S)
+        rec = {"shape": {"num_ranks": cfg.num_ranks, "tokens_per_rank": cfg.tokens_per_rank, "hidden": cfg.hidden,
+                         "num_experts": cfg.num_experts, "num_topk": cfg.num_topk, "use_fp8": cfg.use_fp8},
+               "algorithmic_bytes": alg,
+               "us_at_hbm_peak": {k: round(v / HBM_PEAK_GBPS / 1e3, 2) for k, v in alg.items()}}
+        for label, fused in (("three_launch", 0), ("one_launch", 1)):
+            h = WorldHarness(cfg, device="cuda:0")
+            h.world.set_option("fused_small", fused)
+            h.load(data)
+            h.alloc_dispatch_outputs()
+            h.alloc_combine_io()
+            h.dispatch()
+            h.cast_back()
+            h.combine()
+            torch.cuda.synchronize()
+
+            def step():
+                h.dispatch()
+                h.combine()
+            d_us = time_back_to_back(h.dispatch, iters)
+            c_us = time_back_to_back(h.combine, iters)
+            s_us = time_back_to_back(step, iters)
+            h.dispatch()
+            h.combine()
+            rec[label] = {"dispatch_us": round(d_us, 2), "combine_us": round(c_us, 2), "step_us": round(s_us, 2),
+                          "dispatch_launches": h.world.get_option("last_dispatch_launches"),
+                          "combine_launches": h.world.get_option("last_combine_launches"),
+                          "pct_of_hbm_peak": round((alg["dispatch"] + alg["combine"]) / s_us / 1e3
+                                                   / HBM_PEAK_GBPS * 100, 2)}
+            del h
+        out[name] = rec
+    return out
 
 
 def stream_ceilings(cfg, S, iters):
@@ -575,6 +626,8 @@ def main():
     if not args.no_buffer_api:
         out["buffer_api"] = time_buffer_api(h, args.steps, args.warmup)
         out["buffer_api"]["python_buffer_async_finish"] = time_python_buffer(h, args.steps, args.warmup)
+    if not args.no_small_world:
+        out["small_world"] = time_small_world(max(args.kernel_iters, 100))
     if args.copy_calibration > 0:
         nbytes = args.copy_calibration << 20
         src = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0").fill_(1)

@@ -53,6 +53,13 @@ struct TableChunk {
     uint64_t v[kTableChunk];
 };
 
+// The dispatch rank table of a small world, carried in kernel arguments: v[field * R + rank] with the
+// call's own R (at most kSmallRanks).
+constexpr int kSmallRanks = 8;
+struct SmallTable {
+    uint64_t v[(int)DF_COUNT * kSmallRanks];
+};
+
 // Routing state a dispatch leaves in world-owned device memory.  The world's
 // selections are cut into units of kUnitSelections consecutive (token, k)
 // entries of one rank (units_per_rank per rank, rank-major).  The count kernel
@@ -142,6 +149,10 @@ struct Tuning {
     int combine_nt = 3;        // bit 0: streaming loads, bit 1: streaming stores
     int routing_sum = 1;       // allow the summed routing plan (see UnitPlan) where the shape permits
     int comm_stream = 0;       // 1: per-rank rounds always run on the world's communication stream
+    int fused_small = 1;       // dispatch of a small world (see dispatch_small_kernel) in one launch
+    int fused_small_max = 4096;   // ... when the world names at most this many selections
+    int last_dispatch_launches = 0;   // read-only in spirit: kernels the world's last dispatch / combine call enqueued
+    int last_combine_launches = 0;    // (a rank-table upload counts; launches of other phases' calls do not)
     int blocking = 0;          // 1: a per-rank call returns only when its round has been launched (a thread per rank)
     int block_timeout_ms = 30000;   // how long such a call waits for its peers before it fails
 };
@@ -156,6 +167,10 @@ hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const D
 hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, float* scale_stage,
                        const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
                        hipStream_t stream);
+// The whole dispatch of a small world in one launch (layout, payload, scales, src_info, counts, ranges, and
+// selrow for a combine of the same handle).  The caller has checked: R <= kSmallRanks, d.Tgrid > 0.
+hipError_t launch_dispatch_small(const SmallTable& tb, int32_t* d_selrow, const Dims& d, bool use_fp8, const Tuning& t,
+                                 hipStream_t stream);
 // packed: routes carry (expert, row) instead of a row address
 hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, bool packed, const Dims& d,
                           const Tuning& t, hipStream_t stream);

@@ -493,16 +493,45 @@ __device__ __forceinline__ bool pack_token(const uint64_t* __restrict__ tbl, con
     return true;
 }
 
+// A lane's 16 consecutive bf16 elements (two 16-byte pieces) -> 16 fp8 e4m3 bytes; a 128-element
+// scale group is 8 lanes, whose amax (floor 1e-4, mooncake_ep_kernel.cu:233-264) every lane of
+// the group ends up with.  *scale_inv is the group's stored scale.
+//   NATIVE  false: the arithmetic of the reference's PyTorch statement as CPU PyTorch runs it,
+//           `448.0 / amax` = reciprocal times 448 and `amax / 448.0` a true division
+//           (mooncake_ep_buffer.py:699-702); true: the reference kernel's own, an IEEE
+//           quotient 448 / amax and amax * (1 / 448) (mooncake_ep_kernel.cu:184, :252).
+template <bool NATIVE>
+__device__ __forceinline__ uint4 quantise16(uint4 a, uint4 b, float* scale_inv) {
+    float f[16];
+    const uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        f[2 * j] = bf16_lo(u[j]);
+        f[2 * j + 1] = bf16_hi(u[j]);
+    }
+    float amax = 1e-4f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(f[j]));
+    amax = group_max<8>(amax);
+    // every division here is the compiler's correctly rounded sequence
+    const float scale = NATIVE ? 448.0f / amax : (1.0f / amax) * 448.0f;
+    *scale_inv = NATIVE ? amax * (1.0f / 448.0f) : amax / 448.0f;
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * j] * scale, f[4 * j + 1] * scale, 0, false);
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * j + 2] * scale, f[4 * j + 3] * scale, w, true);
+        o[j] = (uint32_t)w;
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 // fp8: a lane owns 16 consecutive elements (32 B in, 16 B out), a 128-element
 // scale group is 8 lanes.  The group's scales go to the token's row of
 // scale_stage (contiguous); scale_transpose_kernel moves them into the
 // column-major output with coalesced stores (writing them there from here would
 // be 4-byte stores 16 KB apart).
-//   NATIVE  false: the arithmetic of the reference's PyTorch statement as CPU
-//           PyTorch runs it, `448.0 / amax` = reciprocal times 448 and
-//           `amax / 448.0` a true division (mooncake_ep_buffer.py:699-702);
-//           true: the reference kernel's own, an IEEE quotient 448 / amax and
-//           amax * (1 / 448) (mooncake_ep_kernel.cu:184, :252).
+//   NATIVE  which of the reference's two statements of the scale arithmetic (see quantise16)
 template <bool NTL, bool NATIVE>
 __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restrict__ tbl,
                                                         RoutingScratch sc, DispatchSource src,
@@ -539,28 +568,8 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
     const PackDest dst = pack_destination<true>(tbl, sc, idx_row, R, E, K, max_tokens, H, up, r, t, s, lane);
     const int sel_lanes = sel_stride(up, K);   // selection k's destination sits in lane k * sel_lanes
 
-    float f[16];
-    const uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        f[2 * j] = bf16_lo(u[j]);
-        f[2 * j + 1] = bf16_hi(u[j]);
-    }
-    float amax = 1e-4f;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) amax = fmaxf(amax, fabsf(f[j]));
-    amax = group_max<8>(amax);
-    // every division here is the compiler's correctly rounded sequence
-    const float scale = NATIVE ? 448.0f / amax : (1.0f / amax) * 448.0f;
-    const float scale_inv = NATIVE ? amax * (1.0f / 448.0f) : amax / 448.0f;
-    uint32_t o[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        int w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * j] * scale, f[4 * j + 1] * scale, 0, false);
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * j + 2] * scale, f[4 * j + 3] * scale, w, true);
-        o[j] = (uint32_t)w;
-    }
-    const uint4 out = make_uint4(o[0], o[1], o[2], o[3]);
+    float scale_inv;
+    const uint4 out = quantise16<NATIVE>(a, b, &scale_inv);
     if (active && (lane & 7) == 0)
         scale_stage[((int64_t)r * max_tokens + t) * (H >> 7) + (elem0 >> 7)] = scale_inv;
 
@@ -617,6 +626,190 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
 #pragma unroll
         for (int p = 0; p < 2; ++p)
             if (active[p]) store16<false>((void*)(row + off[p]), v[p]);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// dispatch of a small world in one launch
+// ---------------------------------------------------------------------------
+// When the whole world names a few thousand selections (a decode step of one rank, or of a few), the
+// three launches above cost more than the bytes they move: each is close to the floor of an empty
+// kernel.  Here every wave rebuilds the routing it needs by itself, from the ranks' index lists, so one
+// launch does everything - as the reference's dispatch is one launch (mooncake_ep_kernel.cu:138-470).
+// The row of a selection is the number of earlier selections (source rank ascending, then token, then
+// k) that name the same expert: a data wave reads the lists of the earlier ranks and its own rank's up
+// to its token (16-byte loads, two entries per lane, a few KB out of L2) and counts matches for its
+// token's K experts at once.  The first E waves count one expert each over the whole lists and write
+// recv_count and layout_range.  fp8 scales go straight into the column-major layout (4-byte stores 16 KB
+// apart: costly for a large world, nothing next to a launch here).  The rank table travels in the
+// kernel's arguments, so there is no table to upload; nothing is shared between waves, no LDS, no atomics.
+// The slab-0 wave of a token leaves selrow for a combine of the same handle.
+typedef long long i64x2 __attribute__((ext_vector_type(2)));
+
+// counts, per lane, the entries of list[0, n) that equal each of ek[0..KMAX): list and n are wave-uniform;
+// entries outside [0, E) equal nothing (targets are in [0, E) or -2)
+template <int KMAX>
+__device__ __forceinline__ void count_list(uint64_t list, int n, int E, const int (&ek)[KMAX], int (&cnt)[KMAX],
+                                           int lane) {
+    constexpr int kDepth = 4;             // 16-byte loads in flight per lane
+    if ((list & 8) != 0 && n > 0) {
+        // a list that starts in the middle of a 16-byte unit (rank r's slice of a rank-major tensor with an
+        // odd number of entries per rank): its first entry by itself, pairs from there
+        if (lane == 0) {
+            const int64_t v = *(const MCEP_GLOBAL int64_t*)(uintptr_t)list;
+            const int k0 = (uint64_t)v < (uint64_t)E ? (int)v : -1;
+#pragma unroll
+            for (int k = 0; k < KMAX; ++k) cnt[k] += k0 == ek[k] ? 1 : 0;
+        }
+        list += 8;
+        n -= 1;
+    }
+    for (int base = 0; base < n; base += kDepth * 128) {
+        i64x2 v[kDepth];
+#pragma unroll
+        for (int j = 0; j < kDepth; ++j) {
+            const int i = base + j * 128 + 2 * lane;
+            v[j] = i64x2{-1, -1};
+            if (i + 1 < n) v[j] = *(const MCEP_GLOBAL i64x2*)(uintptr_t)(list + (uint64_t)i * 8);
+            else if (i < n) v[j].x = *(const MCEP_GLOBAL int64_t*)(uintptr_t)(list + (uint64_t)i * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < kDepth; ++j) {
+            const int k0 = (uint64_t)v[j].x < (uint64_t)E ? (int)v[j].x : -1;
+            const int k1 = (uint64_t)v[j].y < (uint64_t)E ? (int)v[j].y : -1;
+#pragma unroll
+            for (int k = 0; k < KMAX; ++k) cnt[k] += (k0 == ek[k] ? 1 : 0) + (k1 == ek[k] ? 1 : 0);
+        }
+    }
+}
+
+__device__ __forceinline__ int wave_total(int v) { return __builtin_amdgcn_readlane(wave_scan_inclusive(v), 63); }
+
+// recv_count and layout_range of expert ee, by one wave: its selections in every rank's list
+__device__ __forceinline__ void small_expert(const SmallTable& tb, int R, int E, int K, int max_tokens, int ee) {
+    const int lane = wave_lane();
+    const int L = E / R, q = ee / L, le = ee - q * L;
+    const int64_t RM = (int64_t)R * max_tokens;
+    const int cap = (int)(RM < 0x7fffffff ? RM : 0x7fffffff);   // rows past a block's capacity are dropped
+    const int target[1] = {ee};
+    int run = 0, mine_b = 0, mine_e = 0;
+    for (int rr = 0; rr < R; ++rr) {
+        int c[1] = {0};
+        count_list<1>(tb.v[DF_TOPK_IDX * R + rr], (int)tb.v[DF_NUM_TOKENS * R + rr] * K, E, target, c, lane);
+        const int total = wave_total(c[0]);
+        if (lane == rr) {
+            mine_b = run;
+            mine_e = run + total;
+        }
+        run += total;
+    }
+    const uint64_t recv_x = tb.v[DF_RECV_X * R + q];              // 0: the rank takes no part and receives nothing
+    if (recv_x == 0) return;
+    if (lane == 0) ((int32_t*)tb.v[DF_RECV_COUNT * R + q])[le] = run < cap ? run : cap;
+    if (lane < R) {
+        const int b = mine_b < cap ? mine_b : cap, b2 = mine_e < cap ? mine_e : cap;
+        // count in the low half, begin in the high half; an empty pair is 0
+        ((int64_t*)tb.v[DF_LAYOUT_RANGE * R + q])[(int64_t)le * R + lane] =
+            (b2 > b) ? (((int64_t)b << 32) | (int64_t)(b2 - b)) : 0;
+    }
+}
+
+template <int KMAX, bool FP8, bool NATIVE>
+__global__ __launch_bounds__(256) void dispatch_small_kernel(SmallTable tb, int32_t* __restrict__ selrow, int R, int E,
+                                                              int K, int max_tokens, int H, int slabs, int Tgrid,
+                                                              int total_tasks) {
+    const int lane = wave_lane();
+    int task = __builtin_amdgcn_readfirstlane(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6));
+    if (task >= total_tasks) return;
+    if (task < E) {
+        small_expert(tb, R, E, K, max_tokens, task);
+        return;
+    }
+    task -= E;
+    const int n = task / slabs, s = task - n * slabs;
+    const int r = n / Tgrid, t = n - r * Tgrid;
+    if (t >= (int)tb.v[DF_NUM_TOKENS * R + r]) return;
+    const char* xtok = (const char*)tb.v[DF_X * R + r] + (int64_t)t * H * 2;
+    const uint64_t own_list = tb.v[DF_TOPK_IDX * R + r];
+
+    // the payload loads first: everything below hides behind them
+    constexpr int kSlabBytes = 2048;
+    const int elem0 = s * 1024 + lane * (FP8 ? 16 : 8);          // bf16: the first of two 512-element halves
+    uint4 a = make_uint4(0, 0, 0, 0), b = a;
+    bool act_a, act_b;
+    if (FP8) {
+        act_a = act_b = elem0 < H;
+        if (act_a) {
+            a = load16<false>(xtok + (int64_t)elem0 * 2);
+            b = load16<false>(xtok + (int64_t)elem0 * 2 + 16);
+        }
+    } else {
+        act_a = elem0 < H;
+        act_b = elem0 + 512 < H;
+        if (act_a) a = load16<false>(xtok + (int64_t)elem0 * 2);
+        if (act_b) b = load16<false>(xtok + (int64_t)elem0 * 2 + kSlabBytes / 2);
+    }
+
+    // the token's K experts, one per lane, and each as a wave-uniform target
+    const int li = lane < K ? lane : 0;
+    const int64_t e64 = *(const MCEP_GLOBAL int64_t*)(uintptr_t)(own_list + (uint64_t)((int64_t)t * K + li) * 8);
+    const bool valid = lane < K && (uint64_t)e64 < (uint64_t)E;
+    const int e = valid ? (int)e64 : 0;
+    const int L = E / R, q = e / L, le = e - q * L;
+    // the owner's tensors: asked for as soon as the expert is known, needed after the count
+    const uint64_t base = tb.v[DF_RECV_X * R + q];
+    const uint64_t info = tb.v[DF_SRC_INFO * R + q];
+    const uint64_t sbase = FP8 ? tb.v[DF_RECV_SCALES * R + q] : 0;
+    const int target = valid ? e : -2;
+    int ek[KMAX], cnt[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        ek[k] = __builtin_amdgcn_readlane(target, k);
+        cnt[k] = 0;
+    }
+    // selections of earlier ranks, then of this rank's earlier tokens
+    for (int rr = 0; rr < r; ++rr)
+        count_list<KMAX>(tb.v[DF_TOPK_IDX * R + rr], (int)tb.v[DF_NUM_TOKENS * R + rr] * K, E, ek, cnt, lane);
+    count_list<KMAX>(own_list, t * K, E, ek, cnt, lane);
+    int slot = 0;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+        const int total = wave_total(cnt[k]);
+        // plus the token's own earlier selections of the same expert (a repeated expert gets a row per occurrence)
+        if (lane == k) slot += total;
+        if (lane > k && ek[k] == target) slot += 1;
+    }
+    const int64_t RM = (int64_t)R * max_tokens;
+    const bool ok = valid && slot < RM && base != 0;
+    const int64_t grow = (int64_t)le * RM + slot;
+    uint64_t row = 0, srow = 0;
+    if (ok) {
+        row = base + (uint64_t)grow * (uint64_t)H * (FP8 ? 1 : 2);
+        if (FP8) srow = sbase + (uint64_t)((int64_t)le * (H >> 7) * RM + slot) * 4;
+    }
+    if (s == 0 && lane < K) {
+        // where the selection went, for a combine of this dispatch's handle: expert * R*max + row, or -1
+        selrow[((int64_t)r * max_tokens + t) * K + lane] = ok ? (int)((int64_t)e * RM + slot) : -1;
+        if (ok) ((int32_t*)info)[grow] = t;
+    }
+
+    if (FP8) {
+        float scale_inv;
+        const uint4 out = quantise16<NATIVE>(a, b, &scale_inv);
+        const uint64_t goff = (uint64_t)((int64_t)(elem0 >> 7) * RM) * 4;
+        for (int k = 0; k < K; ++k) {
+            const uint64_t dst = read_lane_u64(row, k);
+            if (dst == 0) continue;
+            if (act_a) store16<false>((void*)(dst + elem0), out);
+            if (act_a && (lane & 7) == 0) *(MCEP_GLOBAL float*)(uintptr_t)(read_lane_u64(srow, k) + goff) = scale_inv;
+        }
+    } else {
+        for (int k = 0; k < K; ++k) {
+            const uint64_t dst = read_lane_u64(row, k);
+            if (dst == 0) continue;
+            if (act_a) store16<false>((void*)(dst + (int64_t)elem0 * 2), a);
+            if (act_b) store16<false>((void*)(dst + (int64_t)elem0 * 2 + kSlabBytes / 2), b);
+        }
     }
 }
 
@@ -1412,6 +1605,33 @@ hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const Di
                        dim3(kTransposeWaves * 64), 0, stream, d_tbl, scale_stage, sc, d.R, d.E, d.H / 128, d.max_tokens,
                        parts, (int)items);
     return hipGetLastError();
+}
+
+template <int KMAX>
+static hipError_t launch_dispatch_small_t(const SmallTable& tb, int32_t* d_selrow, const Dims& d, bool use_fp8,
+                                          const Tuning& t, hipStream_t stream) {
+    const int slabs = (d.H + 1023) / 1024;
+    const long long total = (long long)d.E + (long long)d.R * d.Tgrid * slabs;
+    if (total > 0x7fffffffll) return hipErrorInvalidValue;
+    constexpr int wpb = 4;
+    const dim3 grid((unsigned)((total + wpb - 1) / wpb)), block(wpb * 64);
+#define MCEP_SMALL(FP8, NATIVE)                                                                              \
+    hipLaunchKernelGGL((dispatch_small_kernel<KMAX, FP8, NATIVE>), grid, block, 0, stream, tb, d_selrow, d.R, \
+                       d.E, d.K, d.max_tokens, d.H, slabs, d.Tgrid, (int)total)
+    if (!use_fp8) MCEP_SMALL(false, false);
+    else if (t.fp8_arith == 1) MCEP_SMALL(true, true);
+    else MCEP_SMALL(true, false);
+#undef MCEP_SMALL
+    return hipGetLastError();
+}
+
+hipError_t launch_dispatch_small(const SmallTable& tb, int32_t* d_selrow, const Dims& d, bool use_fp8, const Tuning& t,
+                                 hipStream_t stream) {
+    if (d.R > kSmallRanks || d.Tgrid <= 0 || d_selrow == nullptr) return hipErrorInvalidValue;
+    if (d.K <= 2) return launch_dispatch_small_t<2>(tb, d_selrow, d, use_fp8, t, stream);
+    if (d.K <= 4) return launch_dispatch_small_t<4>(tb, d_selrow, d, use_fp8, t, stream);
+    if (d.K <= 8) return launch_dispatch_small_t<8>(tb, d_selrow, d, use_fp8, t, stream);
+    return launch_dispatch_small_t<16>(tb, d_selrow, d, use_fp8, t, stream);
 }
 
 hipError_t launch_resolve(const uint64_t* d_tbl, CombineRoute* d_routes, uint32_t stamp, bool packed, const Dims& d,

@@ -199,6 +199,7 @@ struct mc_ep_world {
     void* d_zero_row = nullptr;
     std::vector<void*> retired;                   // outgrown scratch, freed with the world
     Tuning tuning;
+    int launches = 0;                             // kernels the call in progress has enqueued (see last_*_launches)
     std::vector<char> silent;
     // per-rank collective bookkeeping
     std::deque<PendingRound<DispatchPost>> dispatch_rounds;
@@ -348,6 +349,7 @@ int upload_table(mc_ep_world* w, int which, const std::vector<uint64_t>& tbl, co
         *d_out = w->d_tbl[which];
         if (w->tbl_cache[which] == tbl) return MC_EP_OK;
         MC_HIP(launch_table_write(w->d_tbl[which], tbl.data(), (int)tbl.size(), stream));
+        w->launches += ((int)tbl.size() + kTableChunk - 1) / kTableChunk;
         w->tbl_cache[which] = tbl;
         return MC_EP_OK;
     }
@@ -457,6 +459,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         MC_ASSERT(recv_scales != nullptr);
     }
     int tgrid = 0;
+    long long selections = 0;
     // the rank table: on the stack, so that the allocation-free variant touches no heap either
     uint64_t tbl[(size_t)DF_COUNT * MC_EP_MAX_QP_COUNT];
     const size_t tbl_words = (size_t)DF_COUNT * R;
@@ -476,8 +479,18 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         tbl[DF_LAYOUT_RANGE * R + r] = layout_range[r];
         tbl[DF_NUM_TOKENS * R + r] = (uint64_t)num_tokens[r];
         if (num_tokens[r] > tgrid) tgrid = num_tokens[r];
+        selections += (long long)num_tokens[r] * num_topk;
     }
+    // A world that names few selections is dispatched in one launch, every wave rebuilding the routing it
+    // needs from the index lists (dispatch_small_kernel); the rank table then travels in kernel arguments.
+    const bool fused = w->tuning.fused_small != 0 && phases == MC_EP_PHASE_ALL && R <= kSmallRanks && tgrid > 0 &&
+                       selections <= (long long)w->tuning.fused_small_max;
     DeviceGuard guard(w->device);
+    w->launches = 0;
+    struct Tally {                                // the option "last_dispatch_launches", on every way out
+        mc_ep_world* w;
+        ~Tally() { w->tuning.last_dispatch_launches = w->launches; }
+    } tally{w};
     // a new dispatch overwrites the staged scales and the routing state: the second part of a round
     // that still waits for its hook has to be enqueued first
     if (!static_scratch && (phases & MC_EP_PHASE_LAYOUT) && w->unfinished)
@@ -485,8 +498,8 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     Dims d{R, num_experts, num_topk, hidden, max_tokens, tgrid};
     plan_units(d, w->tuning);
     // the count kernel keeps per-wave counts and prefixes of every expert in LDS
-    MC_ASSERT(count_lds_bytes(d) <= kMaxCountLdsBytes);
-    MC_ASSERT(d.units() <= kMaxUnits);
+    MC_ASSERT(fused || count_lds_bytes(d) <= kMaxCountLdsBytes);
+    MC_ASSERT(fused || d.units() <= kMaxUnits);
     const size_t UE = (size_t)d.units() * num_experts;
     const size_t stage_floats = use_fp8 ? (size_t)R * max_tokens * (hidden / 128) : 0;
 
@@ -519,7 +532,10 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
                         "dispatch holds " + std::to_string(kStaticScratchBytes) + " (use mc_ep_world_dispatch)");
         // the table travels in kernel arguments on the call's own stream, every time: a recorded call
         // then carries its own copy, and nothing of the world's eager state is involved
-        MC_HIP(launch_table_write(s_tbl, tbl, (int)tbl_words, stream));
+        if (!fused) {
+            MC_HIP(launch_table_write(s_tbl, tbl, (int)tbl_words, stream));
+            w->launches += ((int)tbl_words + kTableChunk - 1) / kTableChunk;
+        }
         d_tbl = s_tbl;
         // the world's own routing state is no longer that of "the last dispatch": combines resolve their handle
         w->last.valid = false;
@@ -527,20 +543,46 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         if (int rc = capture_of(stream, &cap)) return rc;
         RecordingScope recording(cap.active);
         if (int rc = order_begin(w, stream, cap)) return rc;
-        if (int rc = ensure_scratch(w, &w->d_ucount, &w->ucount_cap, UE)) return rc;
-        if (int rc = ensure_scratch(w, &w->d_ubegin, &w->ubegin_cap, UE)) return rc;
-        if (int rc = ensure_scratch(w, &w->d_ucount_t, &w->ucount_t_cap, (size_t)num_experts * kMaxSummedUnits)) return rc;
-        if (int rc = ensure_scratch(w, &w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
         if (int rc = ensure_scratch(w, &w->d_selrow, &w->selrow_cap, (size_t)R * max_tokens * num_topk)) return rc;
-        if (int rc = ensure_scratch(w, &w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
-        if (int rc = ensure_scratch(w, &w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
-        if (stage_floats > 0 && (phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
-            if (int rc = ensure_scale_stage(w, stage_floats)) return rc;
-            stage = w->d_scale_stage;
+        if (!fused) {
+            // (the one-launch dispatch keeps no routing state but selrow, and needs no table in memory)
+            if (int rc = ensure_scratch(w, &w->d_ucount, &w->ucount_cap, UE)) return rc;
+            if (int rc = ensure_scratch(w, &w->d_ubegin, &w->ubegin_cap, UE)) return rc;
+            if (int rc = ensure_scratch(w, &w->d_ucount_t, &w->ucount_t_cap, (size_t)num_experts * kMaxSummedUnits)) return rc;
+            if (int rc = ensure_scratch(w, &w->d_selpos, &w->selpos_cap, (size_t)R * max_tokens * num_topk)) return rc;
+            if (int rc = ensure_scratch(w, &w->d_row_src, &w->row_src_cap, (size_t)num_experts * R * max_tokens)) return rc;
+            if (int rc = ensure_scratch(w, &w->d_counts, &w->counts_cap, (size_t)num_experts)) return rc;
+            if (stage_floats > 0 && (phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
+                if (int rc = ensure_scale_stage(w, stage_floats)) return rc;
+                stage = w->d_scale_stage;
+            }
+            const std::vector<uint64_t> tbl_vec(tbl, tbl + tbl_words);
+            if (int rc = upload_table(w, 0, tbl_vec, cap, stream, &d_tbl)) return rc;
         }
-        const std::vector<uint64_t> tbl_vec(tbl, tbl + tbl_words);
-        if (int rc = upload_table(w, 0, tbl_vec, cap, stream, &d_tbl)) return rc;
         sc = routing_scratch(w);
+    }
+    // what a combine has to know to recognise this dispatch's handle (see mc_ep_world::LastDispatch)
+    auto remember = [&](bool data_done) {
+        auto& ld = w->last;
+        ld.valid = true;
+        ld.hidden = hidden; ld.num_topk = num_topk; ld.max_tokens = max_tokens; ld.num_experts = num_experts;
+        ld.topk_idx.assign(topk_idx, topk_idx + R);
+        ld.recv_x.assign(recv_x, recv_x + R);
+        ld.src_info.assign(src_info, src_info + R);
+        ld.layout_range.assign(layout_range, layout_range + R);
+        ld.num_tokens.assign(num_tokens, num_tokens + R);
+        ld.captured = cap.active;
+        ld.capture_id = cap.id;
+        ld.data_done = data_done;
+        if (cap.active) w->dispatch_captured = true;
+    };
+    if (fused) {
+        SmallTable st{};
+        memcpy(st.v, tbl, tbl_words * sizeof(uint64_t));
+        MC_HIP(launch_dispatch_small(st, sc.selrow, d, use_fp8 != 0, w->tuning, stream));
+        w->launches += 1;
+        if (!static_scratch) remember(true);
+        return MC_EP_OK;
     }
 
     const bool uni = w->tuning.uniform != 0;
@@ -550,24 +592,14 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
     src.tokens = uniform_tokens(num_tokens, R, uni);
     if (phases & MC_EP_PHASE_LAYOUT) {
         MC_HIP(launch_count(d_tbl, sc, src, d, stream));
-        if (!static_scratch) {
-            auto& ld = w->last;
-            ld.valid = true;
-            ld.hidden = hidden; ld.num_topk = num_topk; ld.max_tokens = max_tokens; ld.num_experts = num_experts;
-            ld.topk_idx.assign(topk_idx, topk_idx + R);
-            ld.recv_x.assign(recv_x, recv_x + R);
-            ld.src_info.assign(src_info, src_info + R);
-            ld.layout_range.assign(layout_range, layout_range + R);
-            ld.num_tokens.assign(num_tokens, num_tokens + R);
-            ld.captured = cap.active;
-            ld.capture_id = cap.id;
-            ld.data_done = false;
-            if (cap.active) w->dispatch_captured = true;
-        }
+        w->launches += d.plan.carried ? 1 : 2;    // the prefix pass is a launch of its own unless it rides in pack's
+        if (!static_scratch) remember(false);
     }
-    if ((phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0)
+    if ((phases & (MC_EP_PHASE_DATA | MC_EP_PHASE_FINISH)) && tgrid > 0) {
         MC_HIP(launch_pack(d_tbl, sc, src, stage, d, use_fp8 != 0, w->tuning,
                            (phases & MC_EP_PHASE_DATA) != 0, (phases & MC_EP_PHASE_FINISH) != 0, stream));
+        w->launches += ((phases & MC_EP_PHASE_DATA) ? 1 : 0) + (((phases & MC_EP_PHASE_FINISH) && use_fp8) ? 1 : 0);
+    }
     // under the carried plan the pack launch also produces ubegin and the counts: only now is the
     // routing state complete for a combine to reuse
     if (!static_scratch && (phases & MC_EP_PHASE_DATA)) w->last.data_done = true;
@@ -614,6 +646,11 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
     }
     if (tgrid == 0) return MC_EP_OK;
     DeviceGuard guard(w->device);
+    w->launches = 0;
+    struct Tally {                                // the option "last_combine_launches", on every way out
+        mc_ep_world* w;
+        ~Tally() { w->tuning.last_combine_launches = w->launches; }
+    } tally{w};
     Capture cap;
     if (int rc = capture_of(stream, &cap)) return rc;
     RecordingScope recording(cap.active);
@@ -656,12 +693,16 @@ int world_combine_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_i
             w->stamp += 1;
             // every replay of a recorded call carries the same stamp: clear the routes so that none of an
             // earlier replay passes for this one's
-            if (cap.active)
+            if (cap.active) {
                 MC_HIP(launch_fill_u32(w->d_routes, 0u, (size_t)R * max_tokens * num_topk * (sizeof(CombineRoute) / 4),
                                        stream));
+                w->launches += 1;
+            }
             MC_HIP(launch_resolve(d_tbl, w->d_routes, w->stamp, ps.packed, d, w->tuning, stream));
+            w->launches += 1;
         }
     }
+    if (phases & MC_EP_PHASE_DATA) w->launches += 1;
     if ((phases & MC_EP_PHASE_DATA) && ps.packed)
         MC_HIP(launch_reduce_packed(d_tbl, w->d_routes, w->stamp, routing_scratch(w), direct, src, w->d_zero_row,
                                     ps.factor, ps.scales != nullptr, d, w->tuning, stream));
@@ -1016,6 +1057,10 @@ static int* option_slot(Tuning& t, const char* name) {
     if (!strcmp(name, "routing_sum")) return &t.routing_sum;
     if (!strcmp(name, "combine_waves")) return &t.combine_waves;
     if (!strcmp(name, "combine_nt")) return &t.combine_nt;
+    if (!strcmp(name, "last_dispatch_launches")) return &t.last_dispatch_launches;
+    if (!strcmp(name, "last_combine_launches")) return &t.last_combine_launches;
+    if (!strcmp(name, "fused_small")) return &t.fused_small;
+    if (!strcmp(name, "fused_small_max")) return &t.fused_small_max;
     if (!strcmp(name, "blocking")) return &t.blocking;
     if (!strcmp(name, "block_timeout_ms")) return &t.block_timeout_ms;
     return nullptr;

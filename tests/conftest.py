@@ -25,3 +25,13 @@ def gpu_device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(params=[1, 0], ids=["one_launch", "three_launch"])
+def fused_small(request):
+    """Runs a test once per dispatch path: worlds small enough for the one-launch dispatch take it (1), or
+    take the count / pack / scale-transpose launches like any other world (0)."""
+    from tests import gpu_util
+    gpu_util.DEFAULT_OPTIONS["fused_small"] = request.param
+    yield request.param
+    gpu_util.DEFAULT_OPTIONS.pop("fused_small", None)

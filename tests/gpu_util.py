@@ -15,10 +15,15 @@ def announce(msg: str) -> None:
     sys.stdout.flush()
 
 
+# library options every world made by run_dispatch gets before the test's own (set by the `fused_small`
+# fixture of conftest.py, which runs a test once per dispatch path)
+DEFAULT_OPTIONS: Dict[str, int] = {}
+
+
 def run_dispatch(cfg: EPConfig, data: Dict[str, torch.Tensor], num_tokens: Optional[Sequence[int]] = None,
                  poison: bool = True, present: Optional[Sequence[int]] = None, options: Optional[dict] = None):
     h = WorldHarness(cfg, num_tokens=num_tokens)
-    for k, v in (options or {}).items():
+    for k, v in {**DEFAULT_OPTIONS, **(options or {})}.items():
         h.world.set_option(k, v)
     h.load(data)
     h.alloc_dispatch_outputs(poison=poison)

@@ -53,9 +53,9 @@ def ragged(cfg, on):
 
 @pytest.mark.parametrize("cfg", SMALL, ids=[c.name for c in SMALL])
 @pytest.mark.parametrize("is_ragged", [False, True], ids=["full", "ragged"])
-def test_dispatch_matches_oracle(gpu_device, oracle, cfg, is_ragged):
+def test_dispatch_matches_oracle(gpu_device, oracle, cfg, is_ragged, fused_small):
     nt = ragged(cfg, is_ragged)
-    announce(f"dispatch {cfg} ragged={nt}")
+    announce(f"dispatch {cfg} ragged={nt} fused_small={fused_small}")
     data = generate(cfg, seed=0)
     h = run_dispatch(cfg, data, num_tokens=nt, poison=True)
     ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, cfg.use_fp8)
@@ -65,7 +65,7 @@ def test_dispatch_matches_oracle(gpu_device, oracle, cfg, is_ragged):
 @pytest.mark.parametrize("nt", [0, 1])
 @pytest.mark.parametrize("uniform", [0, 1])
 @pytest.mark.parametrize("arith", [0, 1], ids=["torch_arith", "kernel_arith"])
-def test_fp8_pack_variants_match_oracle(gpu_device, oracle, nt, uniform, arith):
+def test_fp8_pack_variants_match_oracle(gpu_device, oracle, nt, uniform, arith, fused_small):
     """Every tuning variant of the pack path is the same function; the scale arithmetic follows either of the
     reference's two statements of it."""
     cfg = EPConfig("variants", 4, 24, 2560, 16, 3, True)
@@ -88,13 +88,14 @@ def test_dispatch_tuning_options_match_oracle(gpu_device, oracle, opts):
     announce(f"dispatch options {opts}")
     data = generate(cfg, seed=2)
     nt = ragged(cfg, True)
-    h = run_dispatch(cfg, data, num_tokens=nt, poison=True, options=opts)
+    # (these are options of the count / pack / scale-transpose launches: the one-launch dispatch is switched off)
+    h = run_dispatch(cfg, data, num_tokens=nt, poison=True, options={"fused_small": 0, **opts})
     ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, True)
     compare_dispatch(h, ref, check_poison=True)
 
 
 @pytest.mark.parametrize("arith", [0, 1], ids=["torch_arith", "kernel_arith"])
-def test_fp8_every_bf16_value(gpu_device, oracle, arith):
+def test_fp8_every_bf16_value(gpu_device, oracle, arith, fused_small):
     """All finite bf16 bit patterns through the quantiser, in shuffled groups
     (mixed magnitudes) and in sorted groups (tiny amax, subnormal payloads)."""
     bits = torch.arange(0, 65536, dtype=torch.int32)
@@ -132,7 +133,7 @@ def test_fp8_every_bf16_value(gpu_device, oracle, arith):
                            s_ref[si[e, :n].long()].contiguous().view(torch.int32))
 
 
-def test_fp8_inf_and_nan_inputs(gpu_device, oracle):
+def test_fp8_inf_and_nan_inputs(gpu_device, oracle, fused_small):
     H, T = 1024, 8
     g = torch.Generator().manual_seed(2)
     x = torch.randn(T, H, generator=g).to(torch.bfloat16)
@@ -154,7 +155,7 @@ def test_fp8_inf_and_nan_inputs(gpu_device, oracle):
                        ref["scales"][0, 0, :T].contiguous().view(torch.int32))
 
 
-def test_duplicate_experts_follow_the_oracle(gpu_device, oracle):
+def test_duplicate_experts_follow_the_oracle(gpu_device, oracle, fused_small):
     """Out of contract, but defined: one row per (token, k) occurrence; rows that
     would overflow a block's capacity are dropped."""
     cfg = EPConfig("dups", 2, 16, 1024, 4, 4, True)
@@ -187,11 +188,11 @@ COMBINE_CASES = [
 @pytest.mark.parametrize("cfg", COMBINE_CASES, ids=[c.name for c in COMBINE_CASES])
 @pytest.mark.parametrize("is_ragged", [False, True], ids=["full", "ragged"])
 @pytest.mark.parametrize("chunks,cnt,direct", [(1, 3, 1), (2, 3, 1), (1, 0, 1), (1, 3, 0), (2, 0, 0)])
-def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks, cnt, direct):
+def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks, cnt, direct, fused_small):
     """direct=1: the handle is the last dispatch's, rows come from its routing
     state; direct=0: the general path that re-derives rows from the handle."""
     nt = ragged(cfg, is_ragged)
-    announce(f"combine {cfg} ragged={nt} chunks={chunks} nt={cnt} direct={direct}")
+    announce(f"combine {cfg} ragged={nt} chunks={chunks} nt={cnt} direct={direct} fused_small={fused_small}")
     data = generate(cfg, seed=3)
     h = run_dispatch(cfg, data, num_tokens=nt, poison=False,
                      options={"combine_chunks": chunks, "combine_nt": cnt, "combine_direct": direct})
@@ -220,7 +221,7 @@ def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks, cnt,
 
 
 @pytest.mark.parametrize("direct", [1, 0])
-def test_combine_skips_inactive_ranks(gpu_device, oracle, direct):
+def test_combine_skips_inactive_ranks(gpu_device, oracle, direct, fused_small):
     cfg = EPConfig("inactive", 4, 16, 1024, 16, 4, False)
     announce(f"combine with an inactive rank direct={direct}")
     data = generate(cfg, seed=4)
@@ -261,7 +262,7 @@ def test_combine_with_an_older_handle(gpu_device, oracle):
         assert torch.equal(h.combined.cpu().view(torch.int16), want.view(torch.int16))
 
 
-def test_dispatch_with_silent_rank(gpu_device, oracle):
+def test_dispatch_with_silent_rank(gpu_device, oracle, fused_small):
     cfg = EPConfig("silent", 4, 16, 1024, 16, 4, True)
     announce("dispatch with a silent rank")
     data = generate(cfg, seed=5)
@@ -279,7 +280,7 @@ def test_dispatch_with_silent_rank(gpu_device, oracle):
 
 
 @pytest.mark.parametrize("direct", [1, 0])
-def test_ids_outside_the_expert_range_name_no_expert(gpu_device, oracle, direct):
+def test_ids_outside_the_expert_range_name_no_expert(gpu_device, oracle, direct, fused_small):
     """The reference asserts nothing about top-k ids; here anything outside [0, E) is treated like -1 by every
     kernel (and by the oracle), instead of indexing out of bounds."""
     cfg = EPConfig("stray_ids", 4, 24, 512, 8, 4, True)
