@@ -29,18 +29,24 @@ def measured_traffic(workload, kernel):
     profiles/<workload>_hbm_traffic.txt, which `python -m mooncake_amd.benchmarks.hbm_traffic` writes from two
     `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter
     reads for the library's plain copy kernel of known size.  The file records the commit of the library it was
-    measured on, which is passed on; a workload or kernel that was not profiled gives (None, None)."""
+    measured on and a hash of the kernels' sources: (bytes, commit, whether the sources still hash to that).
+    A workload or kernel that was not profiled gives (None, None, None)."""
     path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.txt")
     if not os.path.exists(path):
-        return None, None
-    commit, found = None, None
+        return None, None, None
+    commit, found, sha = None, None, None
     for line in open(path):
         parts = line.split()
         if len(parts) >= 2 and parts[0] == "measured_at_commit":
             commit = parts[1]
+        if len(parts) >= 2 and parts[0] == "kernel_sources_sha256":
+            sha = parts[1]
         if len(parts) >= 3 and parts[0] == "traffic_bytes" and parts[1] == kernel:
             found = int(parts[2])
-    return found, commit
+    # the figure stands only while the kernels' sources are the ones it was measured on
+    from mooncake_amd.benchmarks.hbm_traffic import kernel_sources_sha256
+    current = sha is not None and sha == kernel_sources_sha256()
+    return found, commit, current
 
 
 def parse_args():
@@ -54,6 +60,8 @@ def parse_args():
     ap.add_argument("--no-flushed", action="store_true", help="skip the cache-flushed timing")
     ap.add_argument("--no-buffer-api", action="store_true", help="skip the per-rank Buffer API timing")
     ap.add_argument("--no-small-world", action="store_true", help="skip the launch-bound small-world shapes")
+    ap.add_argument("--small-world", action="store_true",
+                    help="instead of the workload, time only the launch-bound small-world shapes and print them as JSON")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU budget for the cpu_baseline sample")
     ap.add_argument("--kernel-iters", type=int, default=30, help="timed launches per kernel for the roofline figures")
     ap.add_argument("--opt", action="append", default=[], help="library tuning option, name=value")
@@ -460,6 +468,10 @@ def main():
     S = int((data["topk_idx"] >= 0).sum())
     alg = algorithmic_bytes(cfg, S)
 
+    if args.small_world:
+        print(json.dumps({"small_world": time_small_world(max(args.kernel_iters, 100))}))
+        return
+
     if args.stream_ceilings:
         print(json.dumps({"workload": cfg.name, "stream_ceilings": stream_ceilings(cfg, S, args.kernel_iters)}))
         return
@@ -584,7 +596,10 @@ def main():
         # the per-phase loop has (which otherwise lets the GPU run dry for a microsecond or two)
         kernels["reduce"].update(us_in_step=round(c_us, 2))
         achieved = round(alg["combine"] / c_us / 1e3, 1)
-    traffic, traffic_at = measured_traffic(cfg.name, dom)
+    traffic, traffic_at, traffic_current = measured_traffic(cfg.name, dom)
+    if opts or not traffic_current:
+        # measured with other options, or on other kernel sources than the ones running now: not this run's figure
+        traffic = None
     out = {
         "metric": METRIC,
         "value": round(step_gbps, 1),
@@ -619,7 +634,8 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "frac_back_to_back": round(kernels[dom]["bytes"] / kernels[dom]["us_back_to_back"] / 1e3
                                                 / HBM_PEAK_GBPS, 4),
-                     "traffic": None if opts else traffic, "traffic_measured_at_commit": None if opts else traffic_at},
+                     "traffic": traffic, "traffic_measured_at_commit": traffic_at if traffic is not None else None,
+                     "traffic_summary_stale": (traffic_at is not None and not traffic_current) or None},
     }
     if not args.no_flushed:
         out["flushed"] = time_flushed(h, args.kernel_iters, alg)

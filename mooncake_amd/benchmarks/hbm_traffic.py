@@ -23,11 +23,27 @@ import os
 import sys
 from typing import Dict, List
 
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+KERNEL_SOURCES = ("mooncake_amd/csrc/ep_kernels.hip", "mooncake_amd/csrc/ep_kernels.h",
+                  "mooncake_amd/csrc/ep_runtime.hip")
+
+
+def kernel_sources_sha256(root: str = ROOT) -> str:
+    """One hash over the sources the library's kernels and their launch code are built from: a traffic
+    summary records it, and bench.py reports the summary's figures only while the sources still hash to it."""
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(root, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 # kernel-name fragments -> the short names bench.py uses
 KERNELS = [("copy_kernel", "copy"), ("count_kernel", "count"), ("prefix_kernel", "prefix"), ("pack_fp8_kernel", "pack"),
            ("pack_bf16_kernel", "pack"), ("scale_transpose_kernel", "scales"), ("resolve_kernel", "resolve"),
            ("reduce_packed_kernel", "reduce_packed"), ("reduce_kernel", "reduce"), ("cast_chunks_kernel", "cast_chunks"),
-           ("cast_back_kernel", "cast_back")]
+           ("cast_back_kernel", "cast_back"), ("dispatch_small_kernel", "dispatch_small")]
 
 
 def per_kernel_kib(directory: str) -> Dict[str, List[float]]:
@@ -62,6 +78,7 @@ def main(argv=None) -> int:
     f_scale, w_scale = known_kib / mean(fetch["copy"]), known_kib / mean(write["copy"])
     print(f"rocprofv3 counters: HBM traffic per launch, workload {args.workload}")
     print(f"measured_at_commit {args.commit}")
+    print(f"kernel_sources_sha256 {kernel_sources_sha256()}")
     print(f"scale factors from the copy kernel over {args.copy_mib} MiB: FETCH_SIZE x {f_scale:.4f}, "
           f"WRITE_SIZE x {w_scale:.4f}")
     print()
