@@ -96,7 +96,49 @@ def main(argv=None) -> int:
     print()
     for short, total in totals.items():
         print(f"traffic_bytes {short} {total}")
+    print()
+    alg = algorithmic(args.workload)
+    if alg:
+        print("measured / algorithmic bytes per launch (a ratio well above 1 means re-read or partly used sectors):")
+        for short, (nbytes, formula) in alg.items():
+            if short in totals:
+                print(f"  {short:<14}{totals[short] / 1e6:>8.1f} /{nbytes / 1e6:>8.1f} MB = {totals[short] / nbytes:5.3f}   {formula}")
+        print()
+    bench_args = (f"--config {args.workload} --no-cpu-baseline --no-flushed --no-buffer-api --no-small-world --steps 3 "
+                  f"--warmup 1 --kernel-iters 2 --copy-calibration {args.copy_mib}")
+    print("Commands (on the GPU box, from the repository root; cd /tmp && export TMPDIR=/tmp first):")
+    print(f"  rocprofv3 --pmc FETCH_SIZE --output-format csv -d {args.fetch_dir} -o p -- python3 bench.py {bench_args}")
+    print(f"  rocprofv3 --pmc WRITE_SIZE --output-format csv -d {args.write_dir} -o p -- python3 bench.py {bench_args}")
+    print(f"  python3 -m mooncake_amd.benchmarks.hbm_traffic {args.fetch_dir} {args.write_dir} --workload {args.workload} "
+          f"--copy-mib {args.copy_mib} --commit {args.commit}")
+    print("FETCH_SIZE and WRITE_SIZE are in KiB per dispatch; each is scaled by what it reads for the library's plain")
+    print(f"copy kernel over {args.copy_mib} MiB in the same run.  bench.py reports the traffic_bytes line of its dominant")
+    print("kernel as roofline.traffic while the kernel sources still hash to kernel_sources_sha256.")
     return 0
+
+
+def algorithmic(workload: str):
+    """Algorithmic bytes per launch of the data kernels of a named workload (seed 0), with their formulas:
+    N tokens, S valid selections, H hidden, K top-k, E experts, R ranks."""
+    try:
+        from mooncake_amd.workloads import CONFIGS, algorithmic_bytes, generate
+    except ImportError:
+        return {}
+    cfg = CONFIGS.get(workload)
+    if cfg is None:
+        return {}
+    S = int((generate(cfg, seed=0)["topk_idx"] >= 0).sum())
+    N, H = cfg.total_tokens, cfg.hidden
+    alg = algorithmic_bytes(cfg, S)
+    P = H + H // 128 * 4 if cfg.use_fp8 else 2 * H
+    out = {
+        "pack": (alg["dispatch"], "N*H*2 + N*K*8 read; S*(P+4) + E*4 + E*R*8 written (P = H + H/128*4 fp8, 2H bf16; "
+                                  "fp8 scales leave through the scales kernel)"),
+        "reduce": (alg["combine"], "S*H*2 + N*K*12 + S*4 read; N*H*2 written"),
+        "reduce_packed": (S * P + alg["combine"] - S * 2 * H, "S*P + N*K*12 + S*4 read; N*H*2 written"),
+        "cast_back": (S * P + S * 2 * H, "S*P read; S*H*2 written"),
+    }
+    return out
 
 
 if __name__ == "__main__":

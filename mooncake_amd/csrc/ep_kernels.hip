@@ -1071,18 +1071,52 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
     constexpr int kSlab = FP8 ? 1024 : 512;
     constexpr int kLaneElems = kSlab / 64;
     const int lane = wave_lane();
-    // Blocks go round-robin over the 8 XCDs, each with an L2 of its own.  The rows that one source rank
+    // Blocks go round-robin over the 8 XCDs, each with an L2 of its own.  The rows that the source ranks
     // sent to an expert are neighbours in the expert's block, so their scales of one group share 64-byte
-    // sectors: all the waves of a (rank, slab) pair - the ones that read those sectors - are therefore
-    // given to one XCD, next to each other in launch order (group_blocks consecutive blocks of that XCD).
+    // sectors.  group_blocks > 0 (bf16 payloads, which have no scales; option packed_map = 0): all the waves
+    // of a (rank, slab) pair are given to one XCD, next to each other in launch order (group_blocks
+    // consecutive blocks of that XCD).  group_blocks < 0 (fp8): slabs are owned by XCDs, see below.
     const int wpb = blockDim.x >> 6;
     const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
-    const int gl = seq / group_blocks, tb = seq - gl * group_blocks;
-    const int gid = gl * 8 + xcd;
-    if (gid >= R * slabs) return;
-    const int r = gid / slabs, s = gid - r * slabs;
-    const int t = __builtin_amdgcn_readfirstlane(tb * wpb + (threadIdx.x >> 6));
-    if (t >= Tgrid) return;
+    int r, s, t;
+    if (group_blocks > 0) {
+        const int gl = seq / group_blocks, tb = seq - gl * group_blocks;
+        const int gid = gl * 8 + xcd;
+        if (gid >= R * slabs) return;
+        r = gid / slabs;
+        s = gid - r * slabs;
+        t = __builtin_amdgcn_readfirstlane(tb * wpb + (threadIdx.x >> 6));
+        if (t >= Tgrid) return;
+    } else {
+        // Slabs owned by XCDs: every scale of a 128-element group is then read through one XCD's L2 only,
+        // whichever token asks for it, and all XCDs move through the tokens together.  slabs = 8a + b: slab
+        // j of the first 8a belongs to XCD j % 8 for every token; of the other b, slab 8a + c belongs to
+        // m = 8 / b XCDs, which share the tokens of the first b * m residues modulo 8 between them, and the
+        // 8 - b * m XCDs left over take one of the remaining residues each, for all b slabs.  Every XCD
+        // then has P = 8a + b (token residue, slab) pairs per eight consecutive tokens.
+        const int P = -group_blocks;
+        const int w = __builtin_amdgcn_readfirstlane(seq * wpb + (threadIdx.x >> 6));
+        const int o = w / P, i = w - o * P;
+        const int b = slabs & 7, a8 = slabs - b;
+        int rho;
+        if (i < a8) {
+            rho = i & 7;
+            s = xcd + (i & ~7);
+        } else {
+            const int ii = i - a8, m = 8 / b, own = b * m;
+            if (xcd < own) {
+                rho = xcd % m + m * ii;
+                s = a8 + xcd / m;
+            } else {
+                rho = xcd;                  // own + (xcd - own)
+                s = a8 + ii;
+            }
+        }
+        const int n = o * 8 + rho;
+        if (n >= R * Tgrid) return;
+        r = n / Tgrid;
+        t = n - r * Tgrid;
+    }
     const int T = cs.tokens >= 0 ? cs.tokens : (int)tbl[CF_NUM_TOKENS * R + r];
     if (t >= T) return;
     char* orow = (char*)rank_ptr(tbl, cs.out, CF_OUT, R, r) + (int64_t)t * H * 2;
@@ -1712,10 +1746,20 @@ static hipError_t launch_reduce_packed_t(const ReduceLaunch& rl, const float* d_
     const int slabs = (d.H + slab - 1) / slab;
     if (d.Tgrid <= 0) return hipSuccess;
     const int wpb = clamp_waves(t.combine_waves);
-    // (rank, slab) groups, eight at a time (one per XCD), each a run of group_blocks blocks
-    const int group_blocks = (d.Tgrid + wpb - 1) / wpb;
-    const long long rounds = ((long long)d.R * slabs + 7) / 8;
-    const long long blocks = rounds * 8 * group_blocks;
+    int group_blocks;
+    long long blocks;
+    if (FP8 && t.packed_map != 0) {
+        // slabs owned by XCDs (see the kernel): P (token residue, slab) pairs per XCD and eight tokens
+        const int P = slabs;
+        const long long octets = ((long long)d.R * d.Tgrid + 7) / 8;
+        blocks = (octets * P + wpb - 1) / wpb * 8;
+        group_blocks = -P;
+    } else {
+        // (rank, slab) groups, eight at a time (one per XCD), each a run of group_blocks blocks
+        group_blocks = (d.Tgrid + wpb - 1) / wpb;
+        const long long rounds = ((long long)d.R * slabs + 7) / 8;
+        blocks = rounds * 8 * group_blocks;
+    }
     if (blocks > 0x7fffffffll) return hipErrorInvalidValue;
     hipLaunchKernelGGL((reduce_packed_kernel<KMAX, FP8, FACTOR, DIRECT>), dim3((unsigned)blocks), dim3(wpb * 64), 0,
                        stream, rl.d_tbl, rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d_factor, d.R, d.E, d.K,

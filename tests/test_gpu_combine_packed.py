@@ -25,6 +25,12 @@ CASES = [
     EPConfig("one_rank", 1, 36, 1024, 6, 2, True),
     EPConfig("masked_fp8", 8, 64, 1024, 8, 2, True, masked_fraction=0.3),
     EPConfig("zipf_outliers", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05),
+    # slab counts on either side of the 8 XCDs the kernel's block order deals slabs to: 8, 9, 10 and 16 slabs of
+    # 1024 elements (the cases above have 1, 2, 3 and 5; the full-size test below has 7)
+    EPConfig("h8192_fp8", 4, 12, 8192, 16, 4, True),
+    EPConfig("h9216_fp8", 2, 14, 9216, 8, 3, True),
+    EPConfig("h10240_fp8", 4, 9, 10240, 8, 2, True),
+    EPConfig("h16384_fp8", 2, 10, 16384, 8, 4, True),
 ]
 
 
@@ -44,12 +50,14 @@ def oracle_two_step(oracle, cfg, data, nt, factor, active=None):
 @pytest.mark.parametrize("cfg", CASES, ids=[c.name for c in CASES])
 @pytest.mark.parametrize("is_ragged", [False, True], ids=["full", "ragged"])
 @pytest.mark.parametrize("with_factor", [True, False], ids=["factor", "nofactor"])
-@pytest.mark.parametrize("direct", [1, 0], ids=["direct", "handle"])
-def test_packed_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, with_factor, direct):
+@pytest.mark.parametrize("direct,packed_map", [(1, 1), (0, 1), (1, 0)], ids=["direct", "handle", "direct_rank_groups"])
+def test_packed_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, with_factor, direct, packed_map):
+    """packed_map: how the kernel's blocks are dealt to the XCDs (slabs owned by XCDs, or (rank, slab) groups)."""
     nt = ragged(cfg, is_ragged)
-    announce(f"packed combine {cfg} ragged={nt} factor={with_factor} direct={direct}")
+    announce(f"packed combine {cfg} ragged={nt} factor={with_factor} direct={direct} packed_map={packed_map}")
     data = generate(cfg, seed=21)
-    h = run_dispatch(cfg, data, num_tokens=nt, poison=True, options={"combine_direct": direct})
+    h = run_dispatch(cfg, data, num_tokens=nt, poison=True,
+                     options={"combine_direct": direct, "packed_map": packed_map})
     factor = (torch.arange(cfg.num_experts).float() * 0.1 + 1.0) if with_factor else None
     h.alloc_combine_io()
     h.combined.fill_(7.0)
