@@ -156,9 +156,11 @@ struct Tuning {
     int last_combine_launches = 0;    // (a rank-table upload counts; launches of other phases' calls do not)
     int blocking = 0;          // 1: a per-rank call returns only when its round has been launched (a thread per rank)
     int block_timeout_ms = 30000;   // how long such a call waits for its peers before it fails
+    int block_spin_us = 200;        // ... of which this long awake (yielding the core), before it goes to sleep
 };
 
 // Chooses the unit plan for a shape (summed when allowed, the shape permits and there are tokens).
+// (plan_units, count_lds_bytes and cast_back_chunks are host arithmetic: ep_plan.cpp.)
 void plan_units(Dims& d, const Tuning& t);
 
 hipError_t launch_table_write(uint64_t* d_tbl, const uint64_t* h_tbl, int n_words, hipStream_t stream);
@@ -187,6 +189,7 @@ hipError_t launch_reduce_packed(const uint64_t* d_tbl, const CombineRoute* d_rou
                                 const float* d_factor, bool use_fp8, const Dims& d, const Tuning& t, hipStream_t stream);
 // packed rows below packed_recv_count -> bf16 rows times factor[expert]; max_rows bounds the world's valid rows
 // d_chunk_map: 16 bytes x (cast_back_chunks(max_rows, E) + 1) of scratch for the kernel's work list
+constexpr int kCastRows = 4;          // packed rows of one expert per work item of the cast-back kernel
 long long cast_back_chunks(long long max_rows, int num_experts);
 hipError_t launch_cast_back(const uint64_t* d_tbl, void* d_chunk_map, const float* d_factor, bool use_fp8,
                             long long max_rows, const Dims& d, hipStream_t stream);

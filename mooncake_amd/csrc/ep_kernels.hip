@@ -1242,7 +1242,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
 // finds its expert by bisection of the scanned begins.  It costs a launch, and
 // saves every block of the main kernel the same scan (a chain of dependent
 // loads) in front of its first row.
-constexpr int kCastRows = 4;
 constexpr int kCastWaves = 4;        // waves per block of the main kernel: kCastRows / kCastWaves rows each
 constexpr int kCastCols = 1024;
 constexpr int kCastMaxExperts = 4096;
@@ -1538,29 +1537,6 @@ hipError_t launch_clear_words(const uint64_t* h_ptrs, int n_ptrs, int words, hip
     return hipSuccess;
 }
 
-size_t count_lds_bytes(const Dims& d) {
-    return (size_t)(d.plan.selections() / 64) * d.E * (8 + 2) + 64;
-}
-
-void plan_units(Dims& d, const Tuning& t) {
-    const long long per_rank_sel = (long long)d.max_tokens * d.K;
-    const long long big = (per_rank_sel + kBigUnitSelections - 1) / kBigUnitSelections;
-    const size_t big_lds = (size_t)(kBigUnitSelections / 64) * d.E * (8 + 2) + 64;
-    UnitPlan p;
-    if (t.routing_sum != 0 && d.Tgrid > 0 && big * d.R <= kMaxSummedUnits && big_lds <= kMaxCountLdsBytes) {
-        p.per_rank = (int)big;
-        p.shift = 10;
-        p.summed = 1;
-        p.carried = t.routing_sum == 1 ? 1 : 0;
-    } else {
-        p.per_rank = (int)((per_rank_sel + kUnitSelections - 1) / kUnitSelections);
-        p.shift = 8;
-        p.summed = 0;
-    }
-    p.total = d.R * p.per_rank;
-    d.plan = p;
-}
-
 hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, const Dims& d,
                         hipStream_t stream) {
     const size_t lds = count_lds_bytes(d);
@@ -1786,11 +1762,6 @@ hipError_t launch_reduce_packed(const uint64_t* d_tbl, const CombineRoute* d_rou
     MCEP_PK(16);
 #undef MCEP_PK
 #undef MCEP_P4
-}
-
-long long cast_back_chunks(long long max_rows, int num_experts) {
-    // every row is in one chunk, and each expert has at most one partly filled chunk
-    return (max_rows + kCastRows - 1) / kCastRows + num_experts;
 }
 
 hipError_t launch_cast_back(const uint64_t* d_tbl, void* d_chunk_map, const float* d_factor, bool use_fp8,

@@ -6,7 +6,7 @@
 //     recv_count clear + bf16 dispatch + combine, legacy_buffer_perf.cpp:84-146).
 //
 //   ep_native_bench [--ranks R] [--tokens T] [--hidden H] [--experts E] [--topk K]
-//                   [--bf16] [--warmups W] [--iterations N] [--per-rank]
+//                   [--bf16] [--warmups W] [--iterations N] [--per-rank] [--opt name=value ...]
 //
 // With --per-rank it first drives the per-rank Buffer calls (the reference's binding:
 // mc_ep_buffer_dispatch / mc_ep_buffer_combine, one call per rank and collective) in the three
@@ -26,6 +26,7 @@
 #include <cstring>
 #include <string>
 #include <thread>
+#include <utility>
 #include <vector>
 
 #include "mooncake_ep_hip.h"
@@ -52,6 +53,7 @@ namespace {
 struct Args {
     int ranks = 32, tokens = 128, hidden = 7168, experts = 256, topk = 8, warmups = 20, iterations = 30;
     bool fp8 = true, per_rank = false;
+    std::vector<std::pair<std::string, int>> options;   // --opt name=value: options of the world
 };
 
 Args parse(int argc, char** argv) {
@@ -74,6 +76,15 @@ Args parse(int argc, char** argv) {
         else if (f == "--iterations") a.iterations = value();
         else if (f == "--bf16") a.fp8 = false;
         else if (f == "--per-rank") a.per_rank = true;
+        else if (f == "--opt" && i + 1 < argc) {
+            const std::string kv = argv[++i];
+            const size_t eq = kv.find('=');
+            if (eq == std::string::npos) {
+                std::fprintf(stderr, "--opt wants name=value\n");
+                std::exit(2);
+            }
+            a.options.emplace_back(kv.substr(0, eq), std::atoi(kv.c_str() + eq + 1));
+        }
         else {
             std::fprintf(stderr, "unknown flag %s\n", f.c_str());
             std::exit(2);
@@ -240,9 +251,17 @@ int thread_per_rank(mc_ep_world_t* world, std::vector<mc_ep_buffer_t*>& bufs, co
     EP_OK(mc_ep_world_set_option(world, "blocking", 1));
     HIP_OK(hipMemset((void*)p.out_base, 0xFF, (size_t)R * T * H * 2));
     std::vector<int> failed((size_t)R, 0);
+    // where a rank's thread spends a step: inside its dispatch call (and the wait on its event / hook), inside
+    // its combine call, waiting for its stream (microseconds, summed over the steps)
+    std::vector<double> in_dispatch((size_t)R, 0.0), in_combine((size_t)R, 0.0), in_sync((size_t)R, 0.0);
+    const auto now = [] { return std::chrono::steady_clock::now(); };
+    const auto us_since = [](std::chrono::steady_clock::time_point a) {
+        return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - a).count();
+    };
     std::vector<std::thread> threads;
     std::atomic<int> ready{0};
     std::chrono::steady_clock::time_point t0;
+    std::vector<std::chrono::steady_clock::time_point> finished((size_t)R);
     for (int r = 0; r < R; ++r) {
         threads.emplace_back([&, r] {
             hipStream_t mine;
@@ -258,6 +277,7 @@ int thread_per_rank(mc_ep_world_t* world, std::vector<mc_ep_buffer_t*>& bufs, co
                 const int mode = j % 3;   // default, async, hook in turn: every rank the same mode per step
                 mc_ep_event_t* ev = nullptr;
                 mc_ep_hook_t* hk = nullptr;
+                auto mark = now();
                 int rc = mc_ep_buffer_dispatch(bufs[(size_t)r], p.x[(size_t)r], p.idx[(size_t)r], p.active[(size_t)r],
                                                T, H, K, T, E, -1, 0, p.recv16[(size_t)r], 0, p.count[(size_t)r],
                                                p.src[(size_t)r], p.range[(size_t)r], mode == 1, mode == 2, s, &ev, &hk);
@@ -267,6 +287,8 @@ int thread_per_rank(mc_ep_world_t* world, std::vector<mc_ep_buffer_t*>& bufs, co
                 mc_ep_hook_destroy(hk);
                 ev = nullptr;
                 hk = nullptr;
+                in_dispatch[(size_t)r] += us_since(mark);
+                mark = now();
                 if (rc == MC_EP_OK)
                     rc = mc_ep_buffer_combine(bufs[(size_t)r], p.recv16[(size_t)r], p.idx[(size_t)r], p.w[(size_t)r],
                                               p.src[(size_t)r], p.range[(size_t)r], p.active[(size_t)r], L, T, H, K, T,
@@ -279,17 +301,31 @@ int thread_per_rank(mc_ep_world_t* world, std::vector<mc_ep_buffer_t*>& bufs, co
                     std::fprintf(stderr, "rank %d step %d: %s\n", r, j, mc_ep_last_error());
                     failed[(size_t)r] = 1;
                 }
+                in_combine[(size_t)r] += us_since(mark);
+                mark = now();
                 // the next step's dispatch rewrites what this step's combine reads: a rank must not run
                 // ahead of its own stream, exactly as with the reference's buffers
                 if (hipStreamSynchronize(mine) != hipSuccess) failed[(size_t)r] = 1;
+                in_sync[(size_t)r] += us_since(mark);
             }
-            (void)hipStreamDestroy(mine);
+            finished[(size_t)r] = now();
+            (void)hipStreamDestroy(mine);        // (milliseconds for 32 streams: not part of the steps)
         });
     }
     for (auto& t : threads) t.join();
-    const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+    auto last = finished[0];
+    for (int r = 1; r < R; ++r) last = finished[(size_t)r] > last ? finished[(size_t)r] : last;
+    const double us = std::chrono::duration<double, std::micro>(last - t0).count();
     std::printf("thread per rank: %d threads, each on a stream of its own that it waits for after every step: %.0f us "
                 "per bf16 dispatch + combine step\n", R, us / steps);
+    double d = 0.0, c = 0.0, y = 0.0;
+    for (int r = 0; r < R; ++r) {
+        d += in_dispatch[(size_t)r];
+        c += in_combine[(size_t)r];
+        y += in_sync[(size_t)r];
+    }
+    std::printf("  of which a rank's thread spends, on average: %.0f us in its dispatch call, %.0f us in its combine call, "
+                "%.0f us waiting for its stream\n", d / R / steps, c / R / steps, y / R / steps);
     EP_OK(mc_ep_world_set_option(world, "blocking", 0));
     for (int r = 0; r < R; ++r)
         if (failed[(size_t)r]) return 1;
@@ -358,6 +394,7 @@ int main(int argc, char** argv) {
 
     mc_ep_world_t* world = nullptr;
     EP_OK(mc_ep_world_create(R, &world));
+    for (const auto& o : a.options) EP_OK(mc_ep_world_set_option(world, o.first.c_str(), o.second));
     hipStream_t stream;
     HIP_OK(hipStreamCreate(&stream));
     const uint64_t s = (uint64_t)stream;

@@ -8,8 +8,14 @@
 
 #include <hip/hip_runtime.h>
 
+#include <linux/futex.h>
+#include <sched.h>
+#include <sys/syscall.h>
+#include <unistd.h>
+
+#include <atomic>
 #include <chrono>
-#include <condition_variable>
+#include <climits>
 #include <cstdio>
 #include <cstring>
 #include <deque>
@@ -42,12 +48,18 @@ thread_local std::string g_last_error;
 // One lock for the host bookkeeping of every world, buffer, round, event and hook of the process (an
 // EventHandle may outlive its world, so the lock cannot live in the world): entry points take it for as
 // long as they touch that state and enqueue work, not while they wait for a collective's peers or for
-// its results (the short waits of set-up - a world's destruction, scratch that grows - are inside).  g_round_cv is
-// signalled whenever a round has been launched or has failed, for per-rank callers that block until
-// their collective is complete (option "blocking").
+// its results (the short waits of set-up - a world's destruction, scratch that grows - are inside).  Per-rank
+// callers that block until their collective is complete (option "blocking") sleep on their round's own
+// word (Round::published) with the lock given up, and return without taking it again: when a round of 32
+// ranks completes, its 31 sleepers wake side by side instead of queueing for one mutex (which is what a
+// condition variable makes of a broadcast, and took most of a millisecond per step).
 std::mutex g_mu;
-std::condition_variable g_round_cv;
 using Lock = std::unique_lock<std::mutex>;
+
+long futex_call(std::atomic<int>* word, int op, int value, const timespec* timeout) {
+    static_assert(sizeof(std::atomic<int>) == sizeof(int), "the futex word is the atomic's storage");
+    return syscall(SYS_futex, reinterpret_cast<int*>(word), op, value, timeout, nullptr, 0);
+}
 
 int fail(int code, const std::string& msg) {
     g_last_error = msg;
@@ -93,6 +105,44 @@ struct EventPool {
 struct Round {
     bool launched = false;
     std::string failure;          // why the round's launch failed, if it did
+    // For callers that sleep until the round is decided (option "blocking"): 0 while ranks are missing, then
+    // 1 (launched) or 2 (the launch failed; `failure` was written before).  Written once, with the lock held;
+    // read without it.
+    std::atomic<int> published{0};
+    std::atomic<int> sleepers{0};
+    void publish() {
+        published.store(failure.empty() ? 1 : 2, std::memory_order_seq_cst);
+        if (sleepers.load(std::memory_order_seq_cst) > 0) futex_call(&published, FUTEX_WAKE_PRIVATE, INT_MAX, nullptr);
+    }
+    // false: still undecided after `ms` milliseconds.  The first `spin_us` microseconds are spent looking at
+    // the word and offering the core to other threads in turn, not asleep: when every rank's thread is on its
+    // way, the round is decided within tens of microseconds, and putting a thread to sleep and waking it costs
+    // about as much again per thread (more inside a virtual machine).
+    bool wait_published(int ms, int spin_us) {
+        if (published.load(std::memory_order_acquire) != 0) return true;
+        const auto start = std::chrono::steady_clock::now();
+        const auto deadline = start + std::chrono::milliseconds(ms < 0 ? 0 : ms);
+        const auto spin_end = start + std::chrono::microseconds(spin_us < 0 ? 0 : spin_us);
+        while (std::chrono::steady_clock::now() < spin_end) {
+            if (published.load(std::memory_order_acquire) != 0) return true;
+            sched_yield();
+        }
+        sleepers.fetch_add(1, std::memory_order_seq_cst);
+        bool decided = true;
+        while (published.load(std::memory_order_seq_cst) == 0) {
+            const auto left = std::chrono::duration_cast<std::chrono::nanoseconds>(deadline - std::chrono::steady_clock::now());
+            if (left.count() <= 0) {
+                decided = false;
+                break;
+            }
+            timespec ts;
+            ts.tv_sec = (time_t)(left.count() / 1000000000ll);
+            ts.tv_nsec = (long)(left.count() % 1000000000ll);
+            futex_call(&published, FUTEX_WAIT_PRIVATE, 0, &ts);   // returns at once if the word is no longer 0
+        }
+        sleepers.fetch_sub(1, std::memory_order_seq_cst);
+        return decided || published.load(std::memory_order_acquire) != 0;
+    }
     hipEvent_t done = nullptr;
     std::shared_ptr<EventPool> pool;       // where `done` came from and goes back to
     std::vector<hipStream_t> waited;       // streams that already wait for `done`: a second wait adds nothing
@@ -119,6 +169,16 @@ struct Round {
     }
 };
 
+// How a blocking caller (a thread per rank) takes its share of a round's stream hand-offs off the thread
+// that launches the round: it looks at its own stream when it posts (an event recorded there if anything is
+// in flight, for the launch stream to wait on), and makes its own stream wait for the round when it wakes.
+// The launching thread - the last rank to arrive, with every other rank waiting for it - is left with one wait
+// per busy stream instead of a query, a record and two waits per rank.
+struct StreamHandOff {
+    bool by_caller = false;       // the caller did / does its part itself
+    hipEvent_t before = nullptr;  // what the caller's stream held at the call; null: it was idle
+};
+
 struct DispatchPost {
     bool present = false;
     uint64_t x = 0, topk_idx = 0, active_ranks = 0;
@@ -126,6 +186,7 @@ struct DispatchPost {
     uint64_t recv_x = 0, recv_scales = 0, recv_count = 0, src_info = 0, layout_range = 0;
     bool async = false, hook = false;
     hipStream_t stream = nullptr;
+    StreamHandOff hand;
 };
 
 struct CombinePost {
@@ -134,6 +195,7 @@ struct CombinePost {
     int num_tokens = 0, hidden = 0, num_topk = 0, max_tokens = 0, num_experts = 0, timeout_us = -1;
     bool async = false, hook = false;
     hipStream_t stream = nullptr;
+    StreamHandOff hand;
 };
 
 template <typename Post>
@@ -234,6 +296,10 @@ struct mc_ep_buffer {
     int rank = 0;
     int64_t num_ep_buffer_bytes = 0;
     bool p2p_enabled = true;
+    hipEvent_t before = nullptr;    // see StreamHandOff; re-recorded by every blocking call of the rank
+    ~mc_ep_buffer() {
+        if (before) (void)hipEventDestroy(before);
+    }
 };
 
 struct mc_ep_event {
@@ -741,10 +807,18 @@ int fence_before(mc_ep_world* w, const std::vector<Post>& posts, hipStream_t lau
     std::vector<hipStream_t> seen;
     for (const auto& p : posts) {
         if (!p.present || p.stream == launch) continue;
+        if (p.hand.by_caller) {
+            if (p.hand.before) MC_HIP(hipStreamWaitEvent(launch, p.hand.before, 0));
+            continue;
+        }
         bool dup = false;
         for (auto s : seen) dup |= (s == p.stream);
         if (dup) continue;
         seen.push_back(p.stream);
+        // a stream with nothing in flight has nothing to wait for (a rank that waits for its own stream after
+        // every step, as the reference's tests do): asking costs a microsecond of host time, a cross-stream
+        // hand-off about ten of the device's
+        if (hipStreamQuery(p.stream) == hipSuccess) continue;
         // a wait refers to what the event held when the wait was issued, so one event serves every stream
         MC_HIP(hipEventRecord(w->fence, p.stream));
         MC_HIP(hipStreamWaitEvent(launch, w->fence, 0));
@@ -765,9 +839,9 @@ int fence_after(mc_ep_world* w, const std::vector<Post>& posts, hipStream_t laun
         MC_HIP(hipEventRecord(round->done, launch));
     }
     for (const auto& p : posts) {
-        // default mode: the caller's stream waits for the result; async and
-        // hook callers wait through their event / hook
-        if (!p.present || p.async || p.hook) continue;
+        // default mode: the caller's stream waits for the result (a blocking caller sees to that itself
+        // when it wakes); async and hook callers wait through their event / hook
+        if (!p.present || p.async || p.hook || p.hand.by_caller) continue;
         if (int e = round->make_wait(p.stream)) return e;
     }
     round->launched = true;
@@ -894,10 +968,11 @@ bool round_complete(const mc_ep_world* w, const PendingRound<Post>& pr) {
 int drain_dispatch(mc_ep_world* w) {
     while (!w->dispatch_rounds.empty() && round_complete(w, w->dispatch_rounds.front())) {
         int e = launch_dispatch_round(w, w->dispatch_rounds.front());
-        if (e) w->dispatch_rounds.front().state->failure = g_last_error;
+        const std::shared_ptr<Round> state = w->dispatch_rounds.front().state;
+        if (e) state->failure = g_last_error;
         w->dispatch_rounds.pop_front();
         w->dispatch_base++;
-        g_round_cv.notify_all();
+        state->publish();
         if (e) return e;
     }
     return MC_EP_OK;
@@ -906,10 +981,11 @@ int drain_dispatch(mc_ep_world* w) {
 int drain_combine(mc_ep_world* w) {
     while (!w->combine_rounds.empty() && round_complete(w, w->combine_rounds.front())) {
         int e = launch_combine_round(w, w->combine_rounds.front());
-        if (e) w->combine_rounds.front().state->failure = g_last_error;
+        const std::shared_ptr<Round> state = w->combine_rounds.front().state;
+        if (e) state->failure = g_last_error;
         w->combine_rounds.pop_front();
         w->combine_base++;
-        g_round_cv.notify_all();
+        state->publish();
         if (e) return e;
     }
     return MC_EP_OK;
@@ -943,16 +1019,41 @@ int round_not_ready(const Round* round) {
 // Option "blocking": the caller is one of several threads, one per rank, each of which goes on to use its
 // results as soon as its call returns, as a process of the reference does.  The call therefore returns
 // only when the round has been launched (by the thread whose call completed it), so that whatever the
-// caller enqueues next on its stream is ordered behind the round.  Called with the lock held; the
-// wait gives it up.
+// caller enqueues next on its stream is ordered behind the round.  Called with the lock held; a blocking
+// caller gives it up here and comes back without it (what the entry points do afterwards touches nothing
+// that is shared).
 int wait_for_round(mc_ep_world* w, const std::shared_ptr<Round>& round, Lock& lock) {
     if (w->tuning.blocking == 0) return MC_EP_OK;
-    const auto ready = [&] { return round->launched || !round->failure.empty(); };
     const int ms = w->tuning.block_timeout_ms;
-    if (!g_round_cv.wait_for(lock, std::chrono::milliseconds(ms < 0 ? 0 : ms), ready))
+    lock.unlock();
+    if (!round->wait_published(ms, w->tuning.block_spin_us))
         return fail(MC_EP_ERR_PENDING, "Failed: the call waited " + std::to_string(ms) + " ms for the other live ranks "
                                        "of its collective (option block_timeout_ms); it stays posted");
-    if (!round->failure.empty()) return round_not_ready(round.get());
+    if (round->published.load(std::memory_order_acquire) == 2) {
+        lock.lock();                       // `failure` may be appended to by a later second part
+        return round_not_ready(round.get());
+    }
+    return MC_EP_OK;
+}
+
+// A blocking caller's part before the round (see StreamHandOff); with the lock held.
+int hand_off_before(mc_ep_buffer* b, hipStream_t stream, StreamHandOff* hand) {
+    hand->by_caller = true;
+    hand->before = nullptr;
+    if (hipStreamQuery(stream) == hipSuccess) return MC_EP_OK;       // nothing in flight: nothing to wait for
+    if (b->before == nullptr) MC_HIP(hipEventCreateWithFlags(&b->before, hipEventDisableTiming));
+    // the rank's one event serves every round: a wait issued for an earlier round refers to what the event
+    // held then or, if the rank has run ahead and recorded again, to more of the same stream
+    MC_HIP(hipEventRecord(b->before, stream));
+    hand->before = b->before;
+    return MC_EP_OK;
+}
+
+// ... and after it: the default mode's "the caller's stream waits for the result", by the caller, without
+// the lock (the round's event and launch stream were set before the round was published).
+int hand_off_after(const Round* round, hipStream_t stream, bool default_mode) {
+    if (!default_mode || round->launch_stream == stream || round->done == nullptr) return MC_EP_OK;
+    MC_HIP(hipStreamWaitEvent(stream, round->done, 0));
     return MC_EP_OK;
 }
 
@@ -1064,6 +1165,7 @@ static int* option_slot(Tuning& t, const char* name) {
     if (!strcmp(name, "fused_small_max")) return &t.fused_small_max;
     if (!strcmp(name, "blocking")) return &t.blocking;
     if (!strcmp(name, "block_timeout_ms")) return &t.block_timeout_ms;
+    if (!strcmp(name, "block_spin_us")) return &t.block_spin_us;
     return nullptr;
 }
 
@@ -1355,10 +1457,15 @@ int mc_ep_buffer_dispatch(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_p
     p.src_info = src_info_ptr; p.layout_range = layout_range_ptr;
     p.async = async != 0; p.hook = return_recv_hook != 0;
     p.stream = (hipStream_t)compute_stream_ptr;
+    const bool blocking = w->tuning.blocking != 0;
+    if (blocking)
+        if (int e = hand_off_before(b, p.stream, &p.hand)) return e;
     std::shared_ptr<Round> state = pr.state;
 
     if (int e = drain_dispatch(w)) return e;
     if (int e = wait_for_round(w, state, lock)) return e;
+    if (blocking)
+        if (int e = hand_off_after(state.get(), (hipStream_t)compute_stream_ptr, !async && !return_recv_hook)) return e;
     if (async) {
         auto* ev = new mc_ep_event();
         ev->round = state;
@@ -1419,10 +1526,15 @@ int mc_ep_buffer_combine(mc_ep_buffer_t* b, uint64_t x_ptr, uint64_t topk_idx_pt
     p.num_experts = num_experts; p.timeout_us = timeout_us;
     p.async = async != 0; p.hook = return_recv_hook != 0;
     p.stream = (hipStream_t)compute_stream_ptr;
+    const bool blocking = w->tuning.blocking != 0;
+    if (blocking)
+        if (int e = hand_off_before(b, p.stream, &p.hand)) return e;
     std::shared_ptr<Round> state = pr.state;
 
     if (int e = drain_combine(w)) return e;
     if (int e = wait_for_round(w, state, lock)) return e;
+    if (blocking)
+        if (int e = hand_off_after(state.get(), (hipStream_t)compute_stream_ptr, !async && !return_recv_hook)) return e;
     if (async) {
         auto* ev = new mc_ep_event();
         ev->round = state;
