@@ -110,6 +110,12 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+class PendingError(RuntimeError):
+    """MC_EP_ERR_PENDING: a collective was waited on before every live rank had called it - an event or hook of
+    an incomplete round, or a blocking per-rank call that waited `block_timeout_ms` for its peers.  Such a call
+    stays posted: its round is enqueued when the peers arrive, so its tensors must stay alive."""
+
+
 def last_error() -> str:
     msg = lib().mc_ep_last_error()
     return msg.decode("utf-8", "replace") if msg else ""
@@ -127,6 +133,8 @@ def check(rc: int) -> None:
         raise NotImplementedError(msg)
     if rc == ERR_INVALID:
         raise ValueError(msg)          # std::invalid_argument through pybind11
+    if rc == ERR_PENDING:
+        raise PendingError(msg)
     raise RuntimeError(msg)
 
 

@@ -41,6 +41,14 @@ void check(int rc) {
         throw py::error_already_set();
     }
     if (rc == MC_EP_ERR_INVALID) throw std::invalid_argument(msg ? msg : "invalid argument");   // ValueError
+    if (rc == MC_EP_ERR_PENDING) {
+        // a RuntimeError of its own, shared with the ctypes binding: callers tell "not every rank has called
+        // yet" (the call stays posted) from a failure by the type, not by the text
+        const std::string text = msg ? msg : "pending";
+        py::object type = py::module_::import("mooncake_amd._lib").attr("PendingError");
+        PyErr_SetString(type.ptr(), text.c_str());
+        throw py::error_already_set();
+    }
     throw std::runtime_error(msg ? msg : "mooncake_ep_hip: unknown failure");
 }
 
@@ -50,7 +58,6 @@ using I32s = std::vector<int32_t>;
 struct World {
     mc_ep_world_t* h = nullptr;
     int num_ranks = 0;
-    std::atomic<bool> blocking{false};   // option "blocking": per-rank calls wait for their peers, so they must not hold the GIL
     explicit World(int n) : num_ranks(n) { check(mc_ep_world_create(n, &h)); }
     World(const World&) = delete;
     World& operator=(const World&) = delete;
@@ -107,8 +114,9 @@ CallResult wrap(mc_ep_event_t* ev, mc_ep_hook_t* hook, const WorldPtr& world) {
     return r;
 }
 
-// A call that may wait for other Python threads (one per rank, option "blocking") gives up the GIL for
-// its duration; the library reports its failure per thread, so the error text is still this call's.
+// A per-rank call may wait for other Python threads (one per rank, option "blocking" - which can be set
+// through any binding of the C ABI, so nothing here tries to know): it always gives up the GIL for its
+// duration.  The library reports its failure per thread, so the error text is still this call's.
 template <typename F>
 int without_gil(F&& f) {
     py::gil_scoped_release release;
@@ -146,7 +154,7 @@ struct Buffer {
                                          packed_recv_src_info_ptr, packed_recv_layout_range_ptr, async ? 1 : 0,
                                          return_recv_hook ? 1 : 0, compute_stream_ptr, &ev, &hook);
         };
-        check(world->blocking ? without_gil(call) : call());
+        check(without_gil(call));
         return wrap(ev, hook, world);
     }
 
@@ -164,7 +172,7 @@ struct Buffer {
                                         combined_x_ptr, async ? 1 : 0, return_recv_hook ? 1 : 0, compute_stream_ptr,
                                         &ev, &hook);
         };
-        check(world->blocking ? without_gil(call) : call());
+        check(without_gil(call));
         return wrap(ev, hook, world);
     }
 
@@ -297,7 +305,6 @@ PYBIND11_MODULE(_ep, m) {
         .def("set_option",
              [](World& w, const std::string& name, int value) {
                  check(mc_ep_world_set_option(w.h, name.c_str(), value));
-                 if (name == "blocking") w.blocking = value != 0;
              })
         .def("get_option",
              [](const World& w, const std::string& name) {

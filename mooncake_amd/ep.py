@@ -29,6 +29,7 @@ import torch  # noqa: F401
 from . import _lib
 
 MAX_QP_COUNT = 256   # mooncake_ep_configs.cuh:5
+PendingError = _lib.PendingError   # raised by either binding for MC_EP_ERR_PENDING
 
 _native = None
 if os.environ.get("MOONCAKE_AMD_EP_BINDING", "pybind11") != "ctypes":
@@ -84,10 +85,6 @@ class World:
         _lib.check(_lib.lib().mc_ep_world_set_rank_silent(self._h, int(rank), int(bool(silent))))
 
     def set_option(self, name: str, value: int) -> None:
-        if self._native is not None:
-            # through the module, which has to know about "blocking": its per-rank calls then give up the GIL
-            self._native.set_option(name, int(value))
-            return
         _lib.check(_lib.lib().mc_ep_world_set_option(self._h, name.encode(), int(value)))
 
     def get_option(self, name: str) -> int:

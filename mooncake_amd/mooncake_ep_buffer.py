@@ -147,9 +147,10 @@ class Buffer:
             posted.popleft()
 
     def _retain_if_posted(self, exc: RuntimeError, posted: collections.deque, tensors: tuple, kind: int) -> None:
-        """A blocking call that gave up waiting for its peers (option "blocking") has recorded its arguments all
-        the same: the round is enqueued when the peers arrive, so the tensors stay referenced as for any call."""
-        if "stays posted" in str(exc):
+        """A blocking call that gave up waiting for its peers (option "blocking": the one way a dispatch or
+        combine call fails with MC_EP_ERR_PENDING) has recorded its arguments all the same: the round is enqueued
+        when the peers arrive, so the tensors stay referenced as for any call."""
+        if isinstance(exc, ep.PendingError):
             self._retain(posted, tensors, kind)
 
     @staticmethod

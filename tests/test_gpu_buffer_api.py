@@ -16,7 +16,7 @@ import random
 import pytest
 import torch
 
-from mooncake_amd import Buffer, LogicalGroup
+from mooncake_amd import Buffer, LogicalGroup, ep
 from tests import ref_checks as rc
 from tests.gpu_util import announce
 
@@ -229,13 +229,15 @@ def test_collective_rounds_and_pending_errors(gpu_device):
     (xa0, ia0), (xa1, ia1), (xb0, ib0), (xb1, ib1) = mk(), mk(), mk(), mk()
     ra0 = bufs[0].dispatch(xa0, ia0, None, 16, 4, -1, use_fp8=False, async_finish=True)
     rb0 = bufs[0].dispatch(xb0, ib0, None, 16, 4, -1, use_fp8=False, return_recv_hook=True)   # rank 0 runs ahead
-    with pytest.raises(RuntimeError, match="collective"):
+    # MC_EP_ERR_PENDING: a RuntimeError (what the reference's callers catch) of a type of its own
+    with pytest.raises(ep.PendingError, match="collective") as failure:
         ra0[3].current_stream_wait()
-    with pytest.raises(RuntimeError, match="collective"):
+    assert isinstance(failure.value, RuntimeError)
+    with pytest.raises(ep.PendingError, match="collective"):
         rb0[4]()
     ra1 = bufs[1].dispatch(xa1, ia1, None, 16, 4, -1, use_fp8=False)
     ra0[3].current_stream_wait()                                   # round A is complete now
-    with pytest.raises(RuntimeError, match="collective"):
+    with pytest.raises(ep.PendingError, match="collective"):
         rb0[4]()
     rb1 = bufs[1].dispatch(xb1, ib1, None, 16, 4, -1, use_fp8=False)
     rb0[4]()

@@ -8,7 +8,7 @@ import time
 import pytest
 import torch
 
-from mooncake_amd import Buffer, LogicalGroup, spawn_ranks
+from mooncake_amd import Buffer, LogicalGroup, ep, spawn_ranks
 from tests.gpu_util import announce
 from tests.test_gpu_buffer_lifetime import check_rank_dispatch, oracle_world, rank_inputs
 
@@ -114,8 +114,9 @@ def test_a_blocked_call_gives_up_after_the_timeout_and_stays_posted(gpu_device, 
                                         o["src_info"].data_ptr(), o["layout_range"].data_ptr(), False, False, stream)
 
     t0 = time.perf_counter()
-    with pytest.raises(RuntimeError, match="waited 150 ms"):
+    with pytest.raises(ep.PendingError, match="waited 150 ms") as failure:
         post(0)                                            # nobody else is calling
+    assert isinstance(failure.value, RuntimeError)         # what the reference's callers catch
     assert 0.1 < time.perf_counter() - t0 < 5.0
     assert bufs[0].runtime.pending_calls() == (1, 0)      # the call stays posted
     post(1)                                                # completes the round and returns at once
