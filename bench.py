@@ -249,23 +249,27 @@ def time_buffer_api(h, steps, warmup):
 def time_python_buffer(h, steps, warmup):
     """One level up: the Python `Buffer` with the reference wrapper's signature (mooncake_ep_buffer.py:360-535,
     :538-678), which checks its arguments and allocates the five output tensors of every rank's dispatch with
-    torch.empty inside the call.  In the reference each rank pays that in its own process; here one thread pays
-    it for all ranks, so this figure is host-bound and reported for completeness only."""
+    torch.empty inside the call (here: unless an earlier call's outputs have been let go of and can be handed out
+    again).  In the reference each rank pays that in its own process; here one thread pays it for all ranks, so
+    this figure is host-bound and reported for completeness only."""
     import torch
     from mooncake_amd.mooncake_ep_buffer import Buffer, LogicalGroup
     cfg = h.cfg
     R = cfg.num_ranks
     nbytes = Buffer.get_ep_buffer_size_hint(cfg.max_tokens, cfg.hidden, R, cfg.num_experts)
     bufs = [Buffer(LogicalGroup(h.world, r), nbytes) for r in range(R)]
-    expert_out = [h.expert_out[r] for r in range(R)]
+    # each rank's own tensors, as a per-rank caller holds them (slicing the rank-major allocations inside the
+    # loop would add seven tensor-indexing operations, about 1.5 us each, to every rank's step)
+    xs, idx, wts, act = ([t[r] for r in range(R)] for t in (h.x, h.topk_idx, h.topk_weights, h.active_ranks))
+    expert_out, combined = [h.expert_out[r] for r in range(R)], [h.combined[r] for r in range(R)]
 
     def step():
-        res = [bufs[r].dispatch(h.x[r], h.topk_idx[r], h.active_ranks[r], cfg.max_tokens, cfg.num_experts, -1,
+        res = [bufs[r].dispatch(xs[r], idx[r], act[r], cfg.max_tokens, cfg.num_experts, -1,
                                 use_fp8=cfg.use_fp8, async_finish=True) for r in range(R)]
         for r in range(R):
             res[r][3].current_stream_wait()
-        outs = [bufs[r].combine(expert_out[r], h.topk_idx[r], h.topk_weights[r], h.active_ranks[r], -1, res[r][2],
-                                async_finish=True, out=h.combined[r]) for r in range(R)]
+        outs = [bufs[r].combine(expert_out[r], idx[r], wts[r], act[r], -1, res[r][2],
+                                async_finish=True, out=combined[r]) for r in range(R)]
         for r in range(R):
             outs[r][1].current_stream_wait()
     for _ in range(max(2, warmup // 4)):

@@ -16,6 +16,7 @@
 
 #include <atomic>
 #include <cstdint>
+#include <deque>
 #include <functional>
 #include <map>
 #include <memory>
@@ -139,12 +140,27 @@ struct Buffer {
     Buffer& operator=(const Buffer&) = delete;
     ~Buffer() { mc_ep_buffer_destroy(h); }
 
+    // A round's kernels are enqueued by the call of its last rank, from the raw addresses every rank
+    // posted, so a call's tensors must outlive the call: whatever the caller hands over as `keep_alive`
+    // (the reference's tensors_to_record) is held here until the library reports that the call's round
+    // has been enqueued - also when the call itself gave up waiting for its peers (MC_EP_ERR_PENDING:
+    // it stays posted).  kind 0: dispatch, 1: combine.  The GIL is held.
+    std::deque<py::object> kept[2];
+    void retain(int kind, int rc, py::object& keep_alive) {
+        if (keep_alive.is_none() || (rc != MC_EP_OK && rc != MC_EP_ERR_PENDING)) return;
+        kept[kind].push_back(std::move(keep_alive));
+        int pending[2] = {0, 0};
+        if (mc_ep_buffer_pending_calls(h, &pending[0], &pending[1]) != MC_EP_OK) return;
+        while ((long long)kept[kind].size() > pending[kind]) kept[kind].pop_front();
+    }
+    std::pair<int, int> retained() const { return {(int)kept[0].size(), (int)kept[1].size()}; }
+
     CallResult dispatch(uint64_t x_ptr, uint64_t topk_idx_ptr, uint64_t active_ranks_ptr, int num_tokens, int hidden,
                         int num_topk, int num_max_dispatch_tokens_per_rank, int num_experts, int timeout_us,
                         bool use_fp8, uint64_t packed_recv_x_ptr, uint64_t packed_recv_x_scales_ptr,
                         uint64_t packed_recv_count_ptr, uint64_t packed_recv_src_info_ptr,
                         uint64_t packed_recv_layout_range_ptr, bool async, bool return_recv_hook,
-                        uint64_t compute_stream_ptr) {
+                        uint64_t compute_stream_ptr, py::object keep_alive) {
         mc_ep_event_t* ev = nullptr;
         mc_ep_hook_t* hook = nullptr;
         const auto call = [&] {
@@ -154,7 +170,9 @@ struct Buffer {
                                          packed_recv_src_info_ptr, packed_recv_layout_range_ptr, async ? 1 : 0,
                                          return_recv_hook ? 1 : 0, compute_stream_ptr, &ev, &hook);
         };
-        check(without_gil(call));
+        const int rc = without_gil(call);
+        retain(0, rc, keep_alive);
+        check(rc);
         return wrap(ev, hook, world);
     }
 
@@ -162,7 +180,7 @@ struct Buffer {
                        uint64_t layout_range_ptr, uint64_t active_ranks_ptr, int num_local_experts,
                        int num_combined_tokens, int hidden, int num_topk, int num_max_dispatch_tokens_per_rank,
                        int num_experts, int timeout_us, bool zero_copy, uint64_t combined_x_ptr, bool async,
-                       bool return_recv_hook, uint64_t compute_stream_ptr) {
+                       bool return_recv_hook, uint64_t compute_stream_ptr, py::object keep_alive) {
         mc_ep_event_t* ev = nullptr;
         mc_ep_hook_t* hook = nullptr;
         const auto call = [&] {
@@ -172,7 +190,9 @@ struct Buffer {
                                         combined_x_ptr, async ? 1 : 0, return_recv_hook ? 1 : 0, compute_stream_ptr,
                                         &ev, &hook);
         };
-        check(without_gil(call));
+        const int rc = without_gil(call);
+        retain(1, rc, keep_alive);
+        check(rc);
         return wrap(ev, hook, world);
     }
 
@@ -426,8 +446,21 @@ PYBIND11_MODULE(_ep, m) {
         .def("get_ipc_handle", [](const Buffer&) { return std::vector<int32_t>(); })
         .def("sync_nvlink_ipc_handles", [](Buffer&, py::object, py::object) {})
         .def("pending_calls", &Buffer::pending_calls)
-        .def("dispatch", &Buffer::dispatch)
-        .def("combine", &Buffer::combine);
+        .def("retained", &Buffer::retained, "(dispatch, combine) keep_alive objects still held")
+        // the reference's argument lists (ep_py.cpp:43-44), positional; keep_alive is this module's addition
+        .def("dispatch", &Buffer::dispatch, py::arg("x_ptr"), py::arg("topk_idx_ptr"), py::arg("active_ranks_ptr"),
+             py::arg("num_tokens"), py::arg("hidden"), py::arg("num_topk"),
+             py::arg("num_max_dispatch_tokens_per_rank"), py::arg("num_experts"), py::arg("timeout_us"),
+             py::arg("use_fp8"), py::arg("packed_recv_x_ptr"), py::arg("packed_recv_x_scales_ptr"),
+             py::arg("packed_recv_count_ptr"), py::arg("packed_recv_src_info_ptr"),
+             py::arg("packed_recv_layout_range_ptr"), py::arg("async"), py::arg("return_recv_hook"),
+             py::arg("compute_stream_ptr"), py::arg("keep_alive") = py::none())
+        .def("combine", &Buffer::combine, py::arg("x_ptr"), py::arg("topk_idx_ptr"), py::arg("topk_weights_ptr"),
+             py::arg("src_info_ptr"), py::arg("layout_range_ptr"), py::arg("active_ranks_ptr"),
+             py::arg("num_local_experts"), py::arg("num_combined_tokens"), py::arg("hidden"), py::arg("num_topk"),
+             py::arg("num_max_dispatch_tokens_per_rank"), py::arg("num_experts"), py::arg("timeout_us"),
+             py::arg("zero_copy"), py::arg("combined_x_ptr"), py::arg("async"), py::arg("return_recv_hook"),
+             py::arg("compute_stream_ptr"), py::arg("keep_alive") = py::none());
 
     m.def("_benchmark_legacy_buffer",
           [](const py::object& runtime, const LegacyTensors& t, const LegacyConfig& c) {

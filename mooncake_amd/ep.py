@@ -16,6 +16,7 @@ logical ranks of one world.
 """
 from __future__ import annotations
 
+import collections
 import ctypes
 import os
 from ctypes import c_void_p
@@ -310,6 +311,21 @@ class _CtypesBuffer:
         self._h = handle
         self.rank = int(rank)
         self.num_ranks = int(num_ranks)
+        self._kept = (collections.deque(), collections.deque())   # keep_alive objects: dispatch, combine
+
+    def _retain(self, kind: int, rc: int, keep_alive) -> None:
+        """Holds a call's `keep_alive` until the call's round has been enqueued (also for a call that gave up
+        waiting for its peers and stays posted), as the compiled module's Buffer does."""
+        if keep_alive is None or rc not in (_lib.OK, _lib.ERR_PENDING):
+            return
+        kept = self._kept[kind]
+        kept.append(keep_alive)
+        pending = self.pending_calls()[kind]
+        while len(kept) > pending:
+            kept.popleft()
+
+    def retained(self) -> Tuple[int, int]:
+        return len(self._kept[0]), len(self._kept[1])
 
     def __del__(self):
         try:
@@ -368,28 +384,32 @@ class _CtypesBuffer:
                  num_topk: int, num_max_dispatch_tokens_per_rank: int, num_experts: int, timeout_us: int,
                  use_fp8: bool, packed_recv_x_ptr: int, packed_recv_x_scales_ptr: int, packed_recv_count_ptr: int,
                  packed_recv_src_info_ptr: int, packed_recv_layout_range_ptr: int, async_: bool,
-                 return_recv_hook: bool, compute_stream_ptr: int
+                 return_recv_hook: bool, compute_stream_ptr: int, keep_alive=None
                  ) -> Tuple[Optional[object], Optional[Callable[[], None]]]:
         ev, hook = c_void_p(), c_void_p()
-        _lib.check(_lib.lib().mc_ep_buffer_dispatch(
+        rc = (_lib.lib().mc_ep_buffer_dispatch(
             self._h, x_ptr, topk_idx_ptr, active_ranks_ptr, num_tokens, hidden, num_topk,
             num_max_dispatch_tokens_per_rank, num_experts, timeout_us, int(bool(use_fp8)), packed_recv_x_ptr,
             packed_recv_x_scales_ptr, packed_recv_count_ptr, packed_recv_src_info_ptr,
             packed_recv_layout_range_ptr, int(bool(async_)), int(bool(return_recv_hook)), compute_stream_ptr,
             ctypes.byref(ev), ctypes.byref(hook)))
+        self._retain(0, rc, keep_alive)
+        _lib.check(rc)
         return (_CtypesEventHandle(_handle=ev) if ev else None, _RecvHook(hook, self.world) if hook else None)
 
     def combine(self, x_ptr: int, topk_idx_ptr: int, topk_weights_ptr: int, src_info_ptr: int,
                 layout_range_ptr: int, active_ranks_ptr: int, num_local_experts: int, num_combined_tokens: int,
                 hidden: int, num_topk: int, num_max_dispatch_tokens_per_rank: int, num_experts: int,
                 timeout_us: int, zero_copy: bool, combined_x_ptr: int, async_: bool, return_recv_hook: bool,
-                compute_stream_ptr: int) -> Tuple[Optional[object], Optional[Callable[[], None]]]:
+                compute_stream_ptr: int, keep_alive=None) -> Tuple[Optional[object], Optional[Callable[[], None]]]:
         ev, hook = c_void_p(), c_void_p()
-        _lib.check(_lib.lib().mc_ep_buffer_combine(
+        rc = (_lib.lib().mc_ep_buffer_combine(
             self._h, x_ptr, topk_idx_ptr, topk_weights_ptr, src_info_ptr, layout_range_ptr, active_ranks_ptr,
             num_local_experts, num_combined_tokens, hidden, num_topk, num_max_dispatch_tokens_per_rank,
             num_experts, timeout_us, int(bool(zero_copy)), combined_x_ptr, int(bool(async_)),
             int(bool(return_recv_hook)), compute_stream_ptr, ctypes.byref(ev), ctypes.byref(hook)))
+        self._retain(1, rc, keep_alive)
+        _lib.check(rc)
         return (_CtypesEventHandle(_handle=ev) if ev else None, _RecvHook(hook, self.world) if hook else None)
 
 

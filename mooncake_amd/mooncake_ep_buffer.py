@@ -11,7 +11,7 @@ valid (in stream order) once every live rank has made its call.
 """
 from __future__ import annotations
 
-import collections
+import sys
 from typing import Any, Callable, Optional, Tuple, Union
 
 import torch
@@ -30,10 +30,67 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
+_FAST_STREAM = _raw_stream is not None and _raw_device is not None
+
+
 def _native_current_stream_ptr() -> int:
-    if _raw_stream is not None and _raw_device is not None:
+    if _FAST_STREAM:
         return int(_raw_stream(_raw_device()))
     return int(torch.cuda.current_stream().cuda_stream)
+
+
+_storage_use_count = getattr(torch._C, "_storage_Use_Count", None)
+_getrefcount = sys.getrefcount
+_BF16, _I64, _I32, _F32, _FP8 = torch.bfloat16, torch.int64, torch.int32, torch.float32, torch.float8_e4m3fn
+
+
+class _OutputPool:
+    """Dispatch allocates five output tensors per call (reference :446-487).  A caller that has let go of an
+    earlier call's outputs - no name, tuple, handle, view or keep-alive list refers to them any more - cannot
+    tell a recycled tensor from a fresh one, and five `torch.empty` cost more host time than the rest of the
+    call.  So the outputs of earlier calls are offered again, under exactly that condition: every tensor of the
+    set is referenced by nothing but this pool (Python reference count) and its storage by nothing but that
+    tensor (storage use count, which views and dtype reinterpretations raise).  Otherwise the call gets fresh
+    tensors, as in the reference.  Sets are kept per shape, dtype, device and current stream - the caching
+    allocator, too, reuses a freed block only for the stream it was allocated on - and at most `limit` of them,
+    so memory held by the pool stays bounded (a caller that keeps every output alive pools nothing)."""
+
+    limit = 4
+
+    def __init__(self) -> None:
+        self._sets: dict = {}
+
+    @staticmethod
+    def _count(t: torch.Tensor) -> int:
+        return _storage_use_count(t.untyped_storage()._cdata)
+
+    def find(self, key: tuple) -> Optional[list]:
+        """A set of earlier outputs for `key` that nothing refers to any more, or None."""
+        sets = self._sets.get(key)
+        if sets is None or _storage_use_count is None:     # no way to see views of a storage: never recycle
+            return None
+        refs, uses = _getrefcount, _storage_use_count
+        for tensors, baseline in sets:
+            for i in range(len(tensors)):
+                # tensors[i] inside the call: one reference from the list, one from the argument
+                if refs(tensors[i]) != 2 or uses(tensors[i].untyped_storage()._cdata) != baseline[i]:
+                    break
+            else:
+                return list(tensors)                       # the caller's own references
+        return None
+
+    def add(self, key: tuple, tensors: list) -> list:
+        """Fresh outputs join the pool while it has room; returns the caller's own list of them."""
+        if _storage_use_count is not None:
+            sets = self._sets.setdefault(key, [])
+            if len(sets) < self.limit:
+                sets.append((tensors, [self._count(t) for t in tensors]))
+                return list(tensors)
+        return tensors
+
+    def take(self, key: tuple, make: Callable[[], list]) -> list:
+        found = self.find(key)
+        return found if found is not None else self.add(key, make())
 
 
 class LogicalGroup:
@@ -112,7 +169,7 @@ class EventOverlap:
 
     def current_stream_wait(self) -> None:
         assert self.event is not None
-        self.event.current_stream_wait(_native_current_stream_ptr())
+        self.event.current_stream_wait(_raw_stream(_raw_device()) if _FAST_STREAM else _native_current_stream_ptr())
 
     def __enter__(self) -> Any:
         return self
@@ -133,25 +190,11 @@ class Buffer:
         self.runtime = ep.Buffer(self.rank, self.group_size, num_ep_buffer_bytes, disable_p2p, world=world)
         # there is no slow path here: the HIP kernels are the only implementation
         self._use_fallback = False
-        # A round's kernels are enqueued by the call of its last rank, with the raw addresses every
-        # rank posted: the tensors of a call stay referenced here until the runtime reports that the
-        # call's round has been enqueued (however far ahead of its peers this rank runs).
-        self._posted_dispatch = collections.deque()
-        self._posted_combine = collections.deque()
+        # A round's kernels are enqueued by the call of its last rank, from the raw addresses every rank
+        # posted: each call hands its tensors to the runtime (`keep_alive`), which holds them until it
+        # has enqueued the call's round, however far ahead of its peers this rank runs.
+        self._outputs = _OutputPool()
         self.connect()
-
-    def _retain(self, posted: collections.deque, tensors: tuple, kind: int) -> None:
-        posted.append(tensors)
-        pending = self.runtime.pending_calls()[kind]
-        while len(posted) > pending:
-            posted.popleft()
-
-    def _retain_if_posted(self, exc: RuntimeError, posted: collections.deque, tensors: tuple, kind: int) -> None:
-        """A blocking call that gave up waiting for its peers (option "blocking": the one way a dispatch or
-        combine call fails with MC_EP_ERR_PENDING) has recorded its arguments all the same: the round is enqueued
-        when the peers arrive, so the tensors stay referenced as for any call."""
-        if isinstance(exc, ep.PendingError):
-            self._retain(posted, tensors, kind)
 
     @staticmethod
     def _hook_keeping(hook: Optional[Callable], tensors: tuple) -> Optional[Callable]:
@@ -189,58 +232,65 @@ class Buffer:
                  use_fp8: Optional[bool] = None, async_finish: bool = False, return_recv_hook: bool = False,
                  ) -> Tuple[Union[Tuple[torch.Tensor, torch.Tensor], torch.Tensor], torch.Tensor, Tuple,
                             EventOverlap, Callable]:
-        assert x.dim() == 2 and x.is_contiguous()
-        assert x.dtype == torch.bfloat16
-        assert topk_idx.dim() == 2 and topk_idx.is_contiguous()
-        assert topk_idx.dtype == torch.int64
-        assert x.size(0) == topk_idx.size(0)
-        assert x.size(0) <= num_max_dispatch_tokens_per_rank
-        assert x.size(1) % 16 == 0 and x.size(1) % 128 == 0
-        assert num_experts % self.group_size == 0
+        # the reference's checks (:378-393), on each tensor's shape tuple: this wrapper is all host time
+        xs, ts, group_size = x.shape, topk_idx.shape, self.group_size
+        assert len(xs) == 2 and x.is_contiguous()
+        assert x.dtype == _BF16
+        assert len(ts) == 2 and topk_idx.is_contiguous()
+        assert topk_idx.dtype == _I64
+        num_tokens, hidden = xs
+        assert num_tokens == ts[0]
+        assert num_tokens <= num_max_dispatch_tokens_per_rank
+        assert hidden % 16 == 0 and hidden % 128 == 0
+        assert num_experts % group_size == 0
         if active_ranks is None:
             active_ranks = self._default_active_ranks(x.device)
         else:
             assert active_ranks.dim() == 1 and active_ranks.is_contiguous()
-            assert active_ranks.dtype == torch.int32
-            if active_ranks.numel() != self.group_size:
+            assert active_ranks.dtype == _I32
+            if active_ranks.numel() != group_size:
                 active_ranks = self._default_active_ranks(x.device)
         if use_fp8 is None:
             use_fp8 = True
 
-        num_local_experts = num_experts // self.group_size
-        rm = self.group_size * num_max_dispatch_tokens_per_rank
-        hidden = x.size(1)
-        # outputs are not cleared: rows at and beyond packed_recv_count stay unwritten
-        packed_recv_x = torch.empty((num_local_experts, rm, hidden),
-                                    dtype=torch.float8_e4m3fn if use_fp8 else torch.bfloat16, device=x.device)
-        packed_recv_count = torch.empty((num_local_experts,), dtype=torch.int32, device=x.device)
-        packed_recv_src_info = torch.empty((num_local_experts, rm), dtype=torch.int32, device=x.device)
-        packed_recv_layout_range = torch.empty((num_local_experts, self.group_size), dtype=torch.int64,
-                                               device=x.device)
-        packed_recv_x_scales = None
+        num_local_experts = num_experts // group_size
+        rm = group_size * num_max_dispatch_tokens_per_rank
         if use_fp8:
             assert rm % 4 == 0
-            # column-major per expert: [L, H/128, R*max] storage viewed as [L, R*max, H/128]
-            packed_recv_x_scales = torch.empty((num_local_experts, hidden // 128, rm), dtype=torch.float32,
-                                               device=x.device).transpose(1, 2)
+        device = x.device
+        stream_ptr = _native_current_stream_ptr()
+        key = (num_local_experts, rm, hidden, bool(use_fp8), device, stream_ptr)
+        outs = self._outputs.find(key)
+        if outs is None:
+            # outputs are not cleared: rows at and beyond packed_recv_count stay unwritten
+            outs = [torch.empty((num_local_experts, rm, hidden), dtype=_FP8 if use_fp8 else _BF16, device=device),
+                    torch.empty((num_local_experts,), dtype=_I32, device=device),
+                    torch.empty((num_local_experts, rm), dtype=_I32, device=device),
+                    torch.empty((num_local_experts, group_size), dtype=_I64, device=device)]
+            if use_fp8:
+                # column-major per expert: [L, H/128, R*max] storage viewed as [L, R*max, H/128]
+                outs.append(torch.empty((num_local_experts, hidden // 128, rm), dtype=_F32,
+                                        device=device).transpose(1, 2))
+            outs = self._outputs.add(key, outs)
+        if use_fp8:
+            packed_recv_x, packed_recv_count, packed_recv_src_info, packed_recv_layout_range, packed_recv_x_scales = outs
+            scales_ptr = packed_recv_x_scales.data_ptr()
+        else:
+            packed_recv_x, packed_recv_count, packed_recv_src_info, packed_recv_layout_range = outs
+            packed_recv_x_scales, scales_ptr = None, 0
+        del outs
         tensors_to_record = (x, topk_idx, active_ranks, packed_recv_x, packed_recv_x_scales, packed_recv_count,
                              packed_recv_src_info, packed_recv_layout_range)
-        try:
-            event, hook = self.runtime.dispatch(
-                x.data_ptr(), topk_idx.data_ptr(), active_ranks.data_ptr(), x.size(0), hidden, topk_idx.size(1),
-                num_max_dispatch_tokens_per_rank, num_experts, timeout_us, use_fp8, packed_recv_x.data_ptr(),
-                0 if packed_recv_x_scales is None else packed_recv_x_scales.data_ptr(), packed_recv_count.data_ptr(),
-                packed_recv_src_info.data_ptr(), packed_recv_layout_range.data_ptr(), async_finish, return_recv_hook,
-                _native_current_stream_ptr())
-        except RuntimeError as exc:
-            self._retain_if_posted(exc, self._posted_dispatch, tensors_to_record, 0)
-            raise
+        event, hook = self.runtime.dispatch(
+            x.data_ptr(), topk_idx.data_ptr(), active_ranks.data_ptr(), num_tokens, hidden, ts[1],
+            num_max_dispatch_tokens_per_rank, num_experts, timeout_us, use_fp8, packed_recv_x.data_ptr(),
+            scales_ptr, packed_recv_count.data_ptr(), packed_recv_src_info.data_ptr(),
+            packed_recv_layout_range.data_ptr(), async_finish, return_recv_hook, stream_ptr, tensors_to_record)
         handle = (packed_recv_src_info, packed_recv_layout_range, num_max_dispatch_tokens_per_rank, hidden,
                   num_experts)
-        self._retain(self._posted_dispatch, tensors_to_record, 0)
         return ((packed_recv_x, packed_recv_x_scales) if use_fp8 else packed_recv_x, packed_recv_count, handle,
                 EventOverlap(event, tensors_to_record if async_finish else None),
-                self._hook_keeping(hook, tensors_to_record))
+                None if hook is None else self._hook_keeping(hook, tensors_to_record))
 
     # noinspection PyTypeChecker
     def combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
@@ -249,54 +299,55 @@ class Buffer:
                 ) -> Tuple[torch.Tensor, EventOverlap, Callable]:
         if zero_copy:
             raise NotImplementedError(_ZERO_COPY_COMBINE_UNSUPPORTED)
-        assert x.dim() == 3 and x.is_contiguous()
-        assert x.dtype == torch.bfloat16
-        assert topk_idx.dim() == 2 and topk_idx.is_contiguous()
-        assert topk_idx.dtype == torch.int64
-        assert topk_weights.dim() == 2 and topk_weights.is_contiguous()
-        assert topk_weights.dtype == torch.float32
+        # the reference's checks (:554-567, :616-640), on each tensor's shape tuple
+        xs, ts, ws, group_size = x.shape, topk_idx.shape, topk_weights.shape, self.group_size
+        assert len(xs) == 3 and x.is_contiguous()
+        assert x.dtype == _BF16
+        assert len(ts) == 2 and topk_idx.is_contiguous()
+        assert topk_idx.dtype == _I64
+        assert len(ws) == 2 and topk_weights.is_contiguous()
+        assert topk_weights.dtype == _F32
         if active_ranks is None:
             active_ranks = self._default_active_ranks(x.device)
         else:
             assert active_ranks.dim() == 1 and active_ranks.is_contiguous()
-            assert active_ranks.dtype == torch.int32
-            if active_ranks.numel() != self.group_size:
+            assert active_ranks.dtype == _I32
+            if active_ranks.numel() != group_size:
                 active_ranks = self._default_active_ranks(x.device)
         src_info, layout_range, num_max_dispatch_tokens_per_rank, hidden, num_experts = handle
-        assert x.size(0) == num_experts // self.group_size
-        assert x.size(1) == self.group_size * num_max_dispatch_tokens_per_rank
-        assert x.size(2) == hidden
-        assert x.size(2) % 16 == 0 and x.size(2) % 128 == 0
-        assert topk_idx.size() == topk_weights.size()
-        assert topk_weights.size(0) <= num_max_dispatch_tokens_per_rank
-        assert src_info.dim() == 2 and src_info.is_contiguous()
-        assert src_info.dtype == torch.int32
-        assert src_info.size(0) == x.size(0)
-        assert layout_range.dim() == 2 and layout_range.is_contiguous()
-        assert layout_range.dtype == torch.int64
-        assert layout_range.size(0) == num_experts // self.group_size
-        assert layout_range.size(1) == self.group_size
+        num_local_experts = num_experts // group_size
+        ss, ls = src_info.shape, layout_range.shape
+        assert xs[0] == num_local_experts
+        assert xs[1] == group_size * num_max_dispatch_tokens_per_rank
+        assert xs[2] == hidden
+        assert hidden % 16 == 0 and hidden % 128 == 0
+        assert ts == ws
+        num_combined_tokens = ws[0]
+        assert num_combined_tokens <= num_max_dispatch_tokens_per_rank
+        assert len(ss) == 2 and src_info.is_contiguous()
+        assert src_info.dtype == _I32
+        assert ss[0] == xs[0]
+        assert len(ls) == 2 and layout_range.is_contiguous()
+        assert layout_range.dtype == _I64
+        assert ls[0] == num_local_experts
+        assert ls[1] == group_size
         if out is not None:
-            assert out.dim() == 2 and out.is_contiguous()
-            assert out.size(0) == topk_weights.size(0)
-            assert out.size(1) == hidden
-            assert out.dtype == x.dtype
+            os_ = out.shape
+            assert len(os_) == 2 and out.is_contiguous()
+            assert os_[0] == num_combined_tokens
+            assert os_[1] == hidden
+            assert out.dtype == _BF16
             combined_x = out
         else:
-            combined_x = torch.empty((topk_weights.size(0), hidden), dtype=x.dtype, device=x.device)
+            combined_x = torch.empty((num_combined_tokens, hidden), dtype=_BF16, device=x.device)
         tensors_to_record = (x, topk_idx, topk_weights, active_ranks, src_info, layout_range, combined_x)
-        try:
-            event, hook = self.runtime.combine(
-                x.data_ptr(), topk_idx.data_ptr(), topk_weights.data_ptr(), src_info.data_ptr(),
-                layout_range.data_ptr(), active_ranks.data_ptr(), x.size(0), topk_weights.size(0), hidden,
-                topk_weights.size(1), num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy,
-                combined_x.data_ptr(), async_finish, return_recv_hook, _native_current_stream_ptr())
-        except RuntimeError as exc:
-            self._retain_if_posted(exc, self._posted_combine, tensors_to_record, 1)
-            raise
-        self._retain(self._posted_combine, tensors_to_record, 1)
+        event, hook = self.runtime.combine(
+            x.data_ptr(), topk_idx.data_ptr(), topk_weights.data_ptr(), src_info.data_ptr(),
+            layout_range.data_ptr(), active_ranks.data_ptr(), num_local_experts, num_combined_tokens, hidden,
+            ws[1], num_max_dispatch_tokens_per_rank, num_experts, timeout_us, zero_copy,
+            combined_x.data_ptr(), async_finish, return_recv_hook, _native_current_stream_ptr(), tensors_to_record)
         return (combined_x, EventOverlap(event, tensors_to_record if async_finish else None),
-                self._hook_keeping(hook, tensors_to_record))
+                None if hook is None else self._hook_keeping(hook, tensors_to_record))
 
     def get_next_combine_buffer(self, handle: object):
         raise NotImplementedError(_ZERO_COPY_COMBINE_UNSUPPORTED)

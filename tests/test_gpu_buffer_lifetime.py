@@ -90,6 +90,7 @@ def test_rank_runs_four_rounds_ahead_and_drops_its_tensors(gpu_device, oracle):
         junk2 = [torch.full((T, K), 3, dtype=torch.int64, device=gpu_device) for _ in range(4)]
         del junk, junk2
     assert bufs[0].runtime.pending_calls() == (4, 0)
+    assert bufs[0].runtime.retained() == (4, 0)            # the runtime holds the four calls' tensors
     out1 = []
     for j in range(4):
         x, idx, _ = rounds[j][1]
@@ -103,7 +104,7 @@ def test_rank_runs_four_rounds_ahead_and_drops_its_tensors(gpu_device, oracle):
     # the next call of rank 0 lets go of what the finished rounds pinned
     x, idx, _ = rounds[0][0]
     bufs[0].dispatch(x.to(gpu_device), idx.to(gpu_device), None, T, E, -1, use_fp8=False)
-    assert len(bufs[0]._posted_dispatch) == 1
+    assert bufs[0].runtime.retained() == (1, 0)
 
 
 @pytest.mark.parametrize("use_fp8", [True, False], ids=["fp8", "bf16"])

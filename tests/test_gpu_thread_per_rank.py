@@ -111,7 +111,8 @@ def test_a_blocked_call_gives_up_after_the_timeout_and_stays_posted(gpu_device, 
         o = outs[r]
         return bufs[r].runtime.dispatch(x.data_ptr(), idx.data_ptr(), active.data_ptr(), T, H, K, T, E, -1, False,
                                         o["recv_x"].data_ptr(), 0, o["recv_count"].data_ptr(),
-                                        o["src_info"].data_ptr(), o["layout_range"].data_ptr(), False, False, stream)
+                                        o["src_info"].data_ptr(), o["layout_range"].data_ptr(), False, False, stream,
+                                        (x, idx, o))       # keep_alive: what the Python Buffer hands over
 
     t0 = time.perf_counter()
     with pytest.raises(ep.PendingError, match="waited 150 ms") as failure:
@@ -119,9 +120,11 @@ def test_a_blocked_call_gives_up_after_the_timeout_and_stays_posted(gpu_device, 
     assert isinstance(failure.value, RuntimeError)         # what the reference's callers catch
     assert 0.1 < time.perf_counter() - t0 < 5.0
     assert bufs[0].runtime.pending_calls() == (1, 0)      # the call stays posted
+    assert bufs[0].runtime.retained() == (1, 0)           # ... and so do its tensors, although the call failed
     post(1)                                                # completes the round and returns at once
     torch.cuda.synchronize()
     assert bufs[0].runtime.pending_calls() == (0, 0)
+    assert bufs[1].runtime.retained() == (0, 0)
     ref, *_ = oracle_world(oracle, per_rank, T, E, False)
     for r in range(R):
         o = outs[r]
