@@ -5,14 +5,16 @@ on two calls in a row of one world, the second on a smaller input - so whatever
 the first call left in the shared static scratch must not leak into the second.
 Each dispatch is followed by a combine of the handle it produced (the ordinary
 one reuses its dispatch's routing state, the allocation-free one resolves the
-handle), and the two results must be equal as well."""
+handle), and the two results must be equal as well.  Then the property the entry point exists for - the
+driver's free device memory is the same before and after a call of a shape its world has never seen - and a
+recorded call replayed with eager calls of another shape in between, which overwrite the shared array."""
 import pytest
 import torch
 
 from mooncake_amd import _lib, ep
 from mooncake_amd.harness import WorldHarness
 from mooncake_amd.workloads import CONFIGS, EPConfig, generate
-from tests.gpu_util import announce
+from tests.gpu_util import announce, compare_dispatch
 
 pytestmark = pytest.mark.gpu
 
@@ -60,6 +62,82 @@ def test_noalloc_dispatch_matches_dispatch_twice_in_a_row(gpu_device, use_fp8):
     announce(f"noalloc dispatch, second call {small} tokens {nt}")
     _compare(small, world, generate(small, seed=4), num_tokens=nt)
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("cfg", [EPConfig("never_seen_small", 4, 40, 2048, 32, 6, True),       # one launch
+                                 EPConfig("never_seen_large", 16, 96, 2048, 64, 8, True)],    # count, pack, scales
+                         ids=lambda c: c.name)
+def test_noalloc_dispatch_leaves_device_memory_as_it_was(gpu_device, oracle, cfg):
+    """What the entry point is for: a shape its world has never seen costs no device allocation - the free memory
+    the driver reports is the same before and after the call."""
+    announce(f"noalloc dispatch allocates nothing {cfg}")
+    warm = EPConfig("warm", 2, 8, 256, 4, 2, True)          # loads the library's kernels through another world
+    hw = WorldHarness(warm)
+    hw.load(generate(warm, seed=1))
+    hw.alloc_dispatch_outputs()
+    hw.dispatch(noalloc=True)
+    hw.world.set_option("fused_small", 0)
+    hw.dispatch(noalloc=True)
+    torch.cuda.synchronize()
+    data = generate(cfg, seed=5)
+    h = WorldHarness(cfg)                                   # a fresh world: nothing of this shape has been sized
+    h.load(data)
+    h.alloc_dispatch_outputs(poison=True)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    h.dispatch(noalloc=True)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+    ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, True)
+    compare_dispatch(h, ref, check_poison=True)
+
+
+@pytest.mark.parametrize("fused_small", [1, 0], ids=["one_launch", "three_launch"])
+def test_noalloc_dispatch_in_a_graph_with_other_noalloc_calls_between_replays(gpu_device, oracle, fused_small):
+    """A recorded allocation-free dispatch keeps its rank table and scratch in the array every such call on the
+    GPU shares.  An eager call of another shape between two replays overwrites all of it; the replay must not
+    care (its table travels in the recorded kernels' arguments, its scratch is rewritten before it is read)."""
+    cfg = EPConfig("noalloc_graph", 4, 48, 1024, 16, 4, True, masked_fraction=0.2)
+    other_cfg = EPConfig("noalloc_other", 8, 64, 2048, 64, 8, False)
+    announce(f"noalloc dispatch in a graph {cfg} fused_small={fused_small}, eager {other_cfg} between replays")
+    world = ep.World(cfg.num_ranks)
+    world.set_option("fused_small", fused_small)
+    h = WorldHarness(cfg, world=world)
+    h.load(generate(cfg, seed=60))
+    h.alloc_dispatch_outputs(poison=False)
+    other = WorldHarness(other_cfg)
+    other.world.set_option("fused_small", 0)
+    other.load(generate(other_cfg, seed=61))
+    other.alloc_dispatch_outputs(poison=False)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        h.dispatch(noalloc=True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        h.dispatch(noalloc=True)
+    nt = [cfg.tokens_per_rank] * cfg.num_ranks
+    for seed in (62, 63, 64):
+        data = generate(cfg, seed=seed)
+        h.x.copy_(data["x"])
+        h.topk_idx.copy_(data["topk_idx"])
+        h.recv_count.fill_(-1)
+        other.dispatch(noalloc=True)                        # another shape, another world, the same static array
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = oracle.dispatch(data["x"], data["topk_idx"], nt, cfg.max_tokens, cfg.num_experts, True)
+        compare_dispatch(h, ref, check_poison=False)
+    # and the eager call's own result, after a replay rewrote the array under it
+    other.dispatch(noalloc=True)
+    torch.cuda.synchronize()
+    data = generate(other_cfg, seed=61)
+    ref = oracle.dispatch(data["x"], data["topk_idx"], [other_cfg.tokens_per_rank] * other_cfg.num_ranks,
+                          other_cfg.max_tokens, other_cfg.num_experts, False)
+    compare_dispatch(other, ref, check_poison=False)
 
 
 def test_noalloc_dispatch_rejects_what_does_not_fit(gpu_device):
