@@ -4,9 +4,10 @@ Same three modes, signatures, defaults and error conditions as the reference's
 mooncake-ep/benchmarks/ep_benchmark/routing.py (uniform :19-44, k-hot :47-103,
 Zipf :106-146, table :149-153).  Each generator draws from one seeded
 `torch.Generator` in the order the reference's text does (scores, then
-weights).  The tests check the definitions (distinct experts, expected loads,
-error conditions); that a seed reproduces the reference's tensors value for
-value is not tested, because the reference is not run here.
+weights), so a seed gives the reference's tensors value for value on the CPU:
+the tests hold the generators to the definitions (distinct experts, expected
+loads, error conditions) and to vectors written by the reference's own
+generators (tests/golden/routing_vectors.npz).
 """
 from __future__ import annotations
 

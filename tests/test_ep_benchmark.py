@@ -176,3 +176,28 @@ def test_dequantize_fp8_is_payload_times_group_scale():
     assert out.dtype == torch.bfloat16 and out.shape == x.shape
     want = torch.cat([x.float()[..., :128] * 0.5, x.float()[..., 128:] * 2.0], dim=-1).to(torch.bfloat16)
     assert torch.equal(out, want)
+
+
+def test_routing_generators_reproduce_the_reference_value_for_value():
+    """tests/golden/routing_vectors.npz holds what the reference's own generators return for nine
+    (mode, shape, seed) cases (written by tests/golden/make_routing_golden.py, the one place a file of the
+    reference is run); the generators here must give the same indices and the same weight bits on the CPU."""
+    import json
+    import os
+
+    import numpy as np
+    fixture = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "routing_vectors.npz"))
+    cases = sorted(k for k in fixture.files if k.endswith("_args"))
+    assert len(cases) == 9
+    modes = set()
+    for key in cases:
+        args = json.loads(str(fixture[key]))
+        prefix = key[:-len("_args")]
+        idx, weights = routing.ROUTING_MODES[args["mode"]](args["num_tokens"], args["num_experts"], args["top_k"],
+                                                           device=torch.device("cpu"), seed=args["seed"],
+                                                           **args["extra"])
+        assert idx.dtype == torch.int64 and weights.dtype == torch.float32
+        assert np.array_equal(idx.numpy().astype(np.int32), fixture[prefix + "_topk_idx"]), args
+        assert np.array_equal(weights.numpy().view(np.int32), fixture[prefix + "_topk_weights"]), args
+        modes.add(args["mode"])
+    assert modes == {"uniform", "k_hot", "zipf"}
