@@ -92,8 +92,13 @@ int mc_ep_world_num_ranks(const mc_ep_world_t* world);
 int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
 
 /* Options ("pack_waves", "pack_nt", "uniform", "routing_sum", "combine_direct",
- * "combine_chunks", "combine_waves", "combine_nt": tuning knobs for measurement
- * sweeps; "fp8_arith": 0 (default) the fp8 scale arithmetic of the reference's
+ * "combine_chunks", "combine_waves", "combine_nt", "packed_map": tuning knobs
+ * for measurement sweeps; "fused_small": 1 (default) dispatches a world of at
+ * most 8 ranks and "fused_small_max" (default 4096) selections in one kernel
+ * launch, 0 always takes the count / pack / scale-transpose launches;
+ * "last_dispatch_launches", "last_combine_launches": read them to learn how
+ * many kernels the world's last dispatch / combine call enqueued (a rank-table
+ * upload counts); "fp8_arith": 0 (default) the fp8 scale arithmetic of the reference's
  * PyTorch statement as CPU PyTorch runs it - 448.0 / amax as reciprocal times
  * 448, amax / 448.0 a true division (mooncake_ep_buffer.py:699-702) - or 1 the
  * reference kernel's own, 448 / amax as one IEEE division and amax * (1 / 448)
@@ -105,8 +110,9 @@ int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
  * call's round has been launched - by the thread whose call completed it - so
  * that work the caller enqueues next on its stream is ordered behind the
  * round, which is what a thread per rank needs; a call that has waited
- * "block_timeout_ms" (default 30000) for its peers fails with
- * MC_EP_ERR_PENDING and stays posted). */
+ * "block_timeout_ms" (default 30000) for its peers - the first
+ * "block_spin_us" (default 200) of them awake, yielding its core - fails with
+ * MC_EP_ERR_PENDING and stays posted; no order is then imposed on its stream). */
 int mc_ep_world_set_option(mc_ep_world_t* world, const char* name, int value);
 int mc_ep_world_get_option(const mc_ep_world_t* world, const char* name, int* value);
 
@@ -158,7 +164,11 @@ int mc_ep_world_dispatch_noalloc(mc_ep_world_t* world, const uint64_t* x_ptrs, c
  *   x [E/R, R*max, hidden] bf16 (expert outputs held by the rank; 0: the rank
  *   contributes nothing), topk_idx / topk_weights [T_r, num_topk],
  *   src_info / layout_range: the handle returned by that rank's dispatch,
- *   active_ranks [R] int32 (rank r's own view), combined_x [T_r, hidden] bf16. */
+ *   active_ranks [R] int32 (rank r's own view), combined_x [T_r, hidden] bf16.
+ * topk_idx is read as it is when the kernel runs, as in the reference
+ * (mooncake_ep_kernel.cu:719-732): a selection that was set to -1 after the
+ * dispatch (or no longer names the expert it was dispatched to) contributes
+ * nothing, whichever way combine finds its rows. */
 int mc_ep_world_combine(mc_ep_world_t* world, const uint64_t* x_ptrs, const uint64_t* topk_idx_ptrs,
                         const uint64_t* topk_weights_ptrs, const uint64_t* src_info_ptrs,
                         const uint64_t* layout_range_ptrs, const uint64_t* active_ranks_ptrs,

@@ -25,17 +25,32 @@
 //                   (the reference needs two hops, :273-306 then :442-466);
 //                   scale_transpose_kernel then moves the fp8 scales into
 //                   their column-major layout (:457-465).
+//   dispatch_small_kernel  all of the above in one launch for a world of a few
+//                   thousand selections (one deployed rank's decode step): every
+//                   wave rebuilds the routing it needs from the index lists, as
+//                   the reference's dispatch is one launch
+//                   (mooncake_ep_kernel.cu:138-470).
 //   resolve_kernel  combine's handle (src_info, layout_range) -> source row and
 //                   weight of each (token, k) (data flow of
 //                   mooncake_ep_kernel.cu:611-637); only for a handle that is
 //                   not the last dispatch's.
 //   reduce_kernel   per token: fp32 fused multiply-add over its top-k expert
 //                   rows in k order, round to nearest even bf16
-//                   (mooncake_ep_kernel.cu:711-753).
+//                   (mooncake_ep_kernel.cu:711-753); a selection counts while
+//                   topk_idx, as combine is given it, still names the expert
+//                   (:719-732).
 //   cast_chunks_kernel,  the consumer of the packed layout: valid rows back to
 //   cast_back_kernel     bf16, times a per-expert factor
 //                   (per_token_cast_back, mooncake-wheel/tests/ep_test_utils.py:50-53;
 //                   the mock expert of mooncake-ep/tests/test_ep_grid.py:168-173).
+//   reduce_packed_kernel  combine fused with that consumer: reads dispatch's
+//                   payload (fp8 + scales, or bf16) and gives, bit for bit, what
+//                   cast_back_kernel followed by reduce_kernel gives.
+//   stream_kernel,  measurement only: synthetic streams with the read : write
+//   stream_rows_*   mixes and the row geometry of the data kernels, what the
+//                   memory system gives them with nothing else in the way; and
+//                   copy_kernel, the known-size kernel the profiler's byte
+//                   counters are scaled against.
 #include "ep_kernels.h"
 
 namespace mcep {
@@ -1291,10 +1306,13 @@ __global__ __launch_bounds__(1024) void cast_chunks_kernel(const uint64_t* __res
 }
 
 // A block takes one chunk (kCastRows consecutive packed rows of one expert)
-// times kCastCols columns, so only rows below packed_recv_count cost anything.
-// The chunk's scales (column-major in memory: 64 consecutive rows of one group
-// are 256 contiguous bytes) are staged in LDS; then each wave converts its 16
-// rows, 16 payload bytes (FP8) or 32 (bf16 payload) per lane and row.
+// times kCastCols columns, so only rows below packed_recv_count cost anything;
+// each of its kCastWaves waves converts one row of the chunk.  A lane owns two
+// pieces of 8 elements half the block's width apart: per piece 8 payload bytes
+// and one scale (fp8; the scales of a row sit R*max floats apart in the
+// column-major layout, and the four chunks that share their 64-byte sectors
+// run next to each other on one XCD) or 16 payload bytes (bf16), and one
+// 16-byte store that is contiguous across the wave.  No LDS.
 template <bool FP8>
 __global__ __launch_bounds__(kCastWaves * 64) void cast_back_kernel(const uint64_t* __restrict__ tbl,
                                                          const int4* __restrict__ map,
