@@ -508,6 +508,45 @@ __device__ __forceinline__ bool pack_token(const uint64_t* __restrict__ tbl, con
     return true;
 }
 
+// Slabs owned by XCDs.  Blocks go round-robin over the 8 XCDs, each with an L2 of its own, so which block
+// works on which (token, slab) decides which L2 sees a slab's column-major scales: here every scale of a
+// 128-element group passes through one XCD's L2 only, whichever token it belongs to, and all XCDs move
+// through the tokens together.  slabs = 8a + b: slab j of the first 8a belongs to XCD j % 8 for every
+// token; of the other b, slab 8a + c belongs to m = 8 / b XCDs, which share the tokens of the first
+// b * m residues modulo 8 between them, and the 8 - b * m XCDs left over take one of the remaining
+// residues each, for all b slabs.  Every XCD then has P = slabs (token residue, slab) pairs per eight
+// consecutive tokens, so the work is even.  `w` is the wave's number among those of its XCD (`xcd` =
+// block index % 8); false when it is beyond the last token.
+__device__ __forceinline__ bool xcd_owned_task(int xcd, int w, int slabs, int tokens, int* n_out, int* s_out) {
+    const int P = slabs;
+    const int o = w / P, i = w - o * P;
+    const int b = slabs & 7, a8 = slabs - b;
+    int rho, s;
+    if (i < a8) {
+        rho = i & 7;
+        s = xcd + (i & ~7);
+    } else {
+        const int ii = i - a8, m = 8 / b, own = b * m;
+        if (xcd < own) {
+            rho = xcd % m + m * ii;
+            s = a8 + xcd / m;
+        } else {
+            rho = xcd;                  // own + (xcd - own)
+            s = a8 + ii;
+        }
+    }
+    const int n = o * 8 + rho;
+    *n_out = n;
+    *s_out = s;
+    return n < tokens;
+}
+
+// blocks a launch needs for `tokens` tokens of `slabs` slabs each under that order, wpb waves per block
+static long long xcd_owned_blocks(long long tokens, int slabs, int wpb) {
+    const long long octets = (tokens + 7) / 8;
+    return (octets * slabs + wpb - 1) / wpb * 8;
+}
+
 // A lane's 16 consecutive bf16 elements (two 16-byte pieces) -> 16 fp8 e4m3 bytes; a 128-element
 // scale group is 8 lanes, whose amax (floor 1e-4, mooncake_ep_kernel.cu:233-264) every lane of
 // the group ends up with.  *scale_inv is the group's stored scale.
@@ -1090,7 +1129,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
     // sent to an expert are neighbours in the expert's block, so their scales of one group share 64-byte
     // sectors.  group_blocks > 0 (bf16 payloads, which have no scales; option packed_map = 0): all the waves
     // of a (rank, slab) pair are given to one XCD, next to each other in launch order (group_blocks
-    // consecutive blocks of that XCD).  group_blocks < 0 (fp8): slabs are owned by XCDs, see below.
+    // consecutive blocks of that XCD).  group_blocks < 0 (fp8): slabs are owned by XCDs (xcd_owned_task).
     const int wpb = blockDim.x >> 6;
     const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
     int r, s, t;
@@ -1103,32 +1142,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
         t = __builtin_amdgcn_readfirstlane(tb * wpb + (threadIdx.x >> 6));
         if (t >= Tgrid) return;
     } else {
-        // Slabs owned by XCDs: every scale of a 128-element group is then read through one XCD's L2 only,
-        // whichever token asks for it, and all XCDs move through the tokens together.  slabs = 8a + b: slab
-        // j of the first 8a belongs to XCD j % 8 for every token; of the other b, slab 8a + c belongs to
-        // m = 8 / b XCDs, which share the tokens of the first b * m residues modulo 8 between them, and the
-        // 8 - b * m XCDs left over take one of the remaining residues each, for all b slabs.  Every XCD
-        // then has P = 8a + b (token residue, slab) pairs per eight consecutive tokens.
-        const int P = -group_blocks;
+        // slabs owned by XCDs (see xcd_owned_task): a slab's scales are read through one XCD's L2
         const int w = __builtin_amdgcn_readfirstlane(seq * wpb + (threadIdx.x >> 6));
-        const int o = w / P, i = w - o * P;
-        const int b = slabs & 7, a8 = slabs - b;
-        int rho;
-        if (i < a8) {
-            rho = i & 7;
-            s = xcd + (i & ~7);
-        } else {
-            const int ii = i - a8, m = 8 / b, own = b * m;
-            if (xcd < own) {
-                rho = xcd % m + m * ii;
-                s = a8 + xcd / m;
-            } else {
-                rho = xcd;                  // own + (xcd - own)
-                s = a8 + ii;
-            }
-        }
-        const int n = o * 8 + rho;
-        if (n >= R * Tgrid) return;
+        int n;
+        if (!xcd_owned_task(xcd, w, slabs, R * Tgrid, &n, &s)) return;
         r = n / Tgrid;
         t = n - r * Tgrid;
     }
@@ -1743,11 +1760,8 @@ static hipError_t launch_reduce_packed_t(const ReduceLaunch& rl, const float* d_
     int group_blocks;
     long long blocks;
     if (FP8 && t.packed_map != 0) {
-        // slabs owned by XCDs (see the kernel): P (token residue, slab) pairs per XCD and eight tokens
-        const int P = slabs;
-        const long long octets = ((long long)d.R * d.Tgrid + 7) / 8;
-        blocks = (octets * P + wpb - 1) / wpb * 8;
-        group_blocks = -P;
+        blocks = xcd_owned_blocks((long long)d.R * d.Tgrid, slabs, wpb);
+        group_blocks = -1;
     } else {
         // (rank, slab) groups, eight at a time (one per XCD), each a run of group_blocks blocks
         group_blocks = (d.Tgrid + wpb - 1) / wpb;
