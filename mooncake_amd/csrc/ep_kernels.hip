@@ -1114,7 +1114,9 @@ __device__ __forceinline__ uint32_t scale_round_twice(float a, float b, float s,
 // Up to top-8 the register budget is that of eight waves per SIMD: left to itself the compiler spends
 // twice as many on the variant without a factor (to hoist every load), and at four waves per SIMD that
 // variant ran 5 % slower.  (Sixteen rows in flight do not fit that budget.)
-template <int KMAX, bool FP8, bool FACTOR, bool DIRECT>
+//   CH  bf16 payloads only: 16-byte chunks per lane and row, 512 elements apart (two when there are few
+//       rows per token, as in reduce_kernel: half as many waves, each with as many loads in flight)
+template <int KMAX, bool FP8, bool FACTOR, bool DIRECT, int CH = 1>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ? 8 : 4, 8))) void reduce_packed_kernel(const uint64_t* __restrict__ tbl,
                                                              const CombineRoute* __restrict__ routes, uint32_t stamp,
                                                              RoutingScratch sc, CombineSource cs,
@@ -1122,8 +1124,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
                                                              const float* __restrict__ factor, int R, int E, int K,
                                                              int max_tokens, int H, int slabs, int Tgrid,
                                                              int group_blocks) {
-    constexpr int kSlab = FP8 ? 1024 : 512;
-    constexpr int kLaneElems = kSlab / 64;
+    static_assert(!FP8 || CH == 1, "an fp8 payload is one 16-byte chunk of 16 elements per lane");
+    constexpr int kSlab = FP8 ? 1024 : 512 * CH;
+    constexpr int kChunkElems = FP8 ? 16 : 8;          // elements in a lane's 16-byte chunk
     const int lane = wave_lane();
     // Blocks go round-robin over the 8 XCDs, each with an L2 of its own.  The rows that the source ranks
     // sent to an expert are neighbours in the expert's block, so their scales of one group share 64-byte
@@ -1196,17 +1199,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
         }
     }
 
-    const int elem = s * kSlab + lane * kLaneElems;
-    const bool on = elem < H;
-    const int64_t poff = on ? (int64_t)elem * (FP8 ? 1 : 2) : 0;
-    const int group = on ? (elem >> 7) : 0;
+    int elem[CH];
+    bool on[CH];
+    int64_t poff[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        elem[c] = s * kSlab + c * 512 + lane * kChunkElems;
+        on[c] = elem[c] < H;
+        poff[c] = on[c] ? (int64_t)elem[c] * (FP8 ? 1 : 2) : 0;
+    }
+    const int group = on[0] ? (elem[0] >> 7) : 0;
 
-    uint4 v[KMAX];
+    uint4 v[KMAX][CH];
     float sv[KMAX], wk[KMAX], fk[KMAX];
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
         const uint64_t p = read_lane_u64(src, k);
-        v[k] = load16<true>((const void*)(p + poff));
+#pragma unroll
+        for (int c = 0; c < CH; ++c) v[k][c] = load16<true>((const void*)(p + poff[c]));
         if (FP8) {
             const uint64_t sp = read_lane_u64(ssrc, k);
             const int st = __builtin_amdgcn_readlane(sstride, k);
@@ -1226,16 +1236,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
         fk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), k));
         wk[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k));
         if (DIRECT && __builtin_amdgcn_readlane(live, k) == 0) {
-            v[k] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) v[k][c] = make_uint4(0, 0, 0, 0);
             sv[k] = 0.0f;
         }
     }
-    float acc[kLaneElems];
 #pragma unroll
-    for (int j = 0; j < kLaneElems; ++j) acc[j] = 0.0f;
+    for (int c = 0; c < CH; ++c) {
+    float acc[kChunkElems];
+#pragma unroll
+    for (int j = 0; j < kChunkElems; ++j) acc[j] = 0.0f;
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) {
-        const uint32_t u[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+        const uint32_t u[4] = {v[k][c].x, v[k][c].y, v[k][c].z, v[k][c].w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             if (FP8) {
@@ -1259,12 +1272,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(KMAX <= 8 ?
             }
         }
     }
-    if (!on) return;
-    uint32_t o[kLaneElems / 2];
+    if (!on[c]) continue;
+    uint32_t o[kChunkElems / 2];
 #pragma unroll
-    for (int j = 0; j < kLaneElems / 2; ++j) o[j] = pack_bf16_rne(acc[2 * j], acc[2 * j + 1]);
-    store16<true>(orow + (int64_t)elem * 2, make_uint4(o[0], o[1], o[2], o[3]));
-    if constexpr (FP8) store16<true>(orow + (int64_t)elem * 2 + 16, make_uint4(o[4], o[5], o[6], o[7]));
+    for (int j = 0; j < kChunkElems / 2; ++j) o[j] = pack_bf16_rne(acc[2 * j], acc[2 * j + 1]);
+    store16<true>(orow + (int64_t)elem[c] * 2, make_uint4(o[0], o[1], o[2], o[3]));
+    if constexpr (FP8) store16<true>(orow + (int64_t)elem[c] * 2 + 16, make_uint4(o[4], o[5], o[6], o[7]));
+    }
 }
 
 // Work list of the cast-back kernel: which (expert, row chunk) each chunk
@@ -1750,10 +1764,10 @@ hipError_t launch_reduce(const uint64_t* d_tbl, const CombineRoute* d_routes, ui
 #undef MCEP_K
 }
 
-template <int KMAX, bool FP8, bool FACTOR, bool DIRECT>
+template <int KMAX, bool FP8, bool FACTOR, bool DIRECT, int CH = 1>
 static hipError_t launch_reduce_packed_t(const ReduceLaunch& rl, const float* d_factor, const Dims& d, const Tuning& t,
                                          hipStream_t stream) {
-    const int slab = FP8 ? 1024 : 512;
+    const int slab = FP8 ? 1024 : 512 * CH;
     const int slabs = (d.H + slab - 1) / slab;
     if (d.Tgrid <= 0) return hipSuccess;
     const int wpb = clamp_waves(t.combine_waves);
@@ -1769,7 +1783,7 @@ static hipError_t launch_reduce_packed_t(const ReduceLaunch& rl, const float* d_
         blocks = rounds * 8 * group_blocks;
     }
     if (blocks > 0x7fffffffll) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((reduce_packed_kernel<KMAX, FP8, FACTOR, DIRECT>), dim3((unsigned)blocks), dim3(wpb * 64), 0,
+    hipLaunchKernelGGL((reduce_packed_kernel<KMAX, FP8, FACTOR, DIRECT, CH>), dim3((unsigned)blocks), dim3(wpb * 64), 0,
                        stream, rl.d_tbl, rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d_factor, d.R, d.E, d.K,
                        d.max_tokens, d.H, slabs, d.Tgrid, group_blocks);
     return hipGetLastError();
@@ -1788,6 +1802,14 @@ hipError_t launch_reduce_packed(const uint64_t* d_tbl, const CombineRoute* d_rou
         if (use_fp8) return fac ? MCEP_P4(KMAX, true, true) : MCEP_P4(KMAX, true, false);            \
         return fac ? MCEP_P4(KMAX, false, true) : MCEP_P4(KMAX, false, false);                       \
     } while (0)
+    // a bf16 payload with few rows per token: two chunks per lane, as in the combine kernel
+#define MCEP_P2(KMAX, FACTOR)                                                                        \
+    (direct ? launch_reduce_packed_t<KMAX, false, FACTOR, true, 2>(rl, d_factor, d, t, stream)       \
+            : launch_reduce_packed_t<KMAX, false, FACTOR, false, 2>(rl, d_factor, d, t, stream))
+    const int ch = t.combine_chunks > 0 ? (t.combine_chunks >= 2 ? 2 : 1) : (d.K <= 4 ? 2 : 1);
+    if (!use_fp8 && ch == 2 && d.K <= 2) return fac ? MCEP_P2(2, true) : MCEP_P2(2, false);
+    if (!use_fp8 && ch == 2 && d.K <= 4) return fac ? MCEP_P2(4, true) : MCEP_P2(4, false);
+#undef MCEP_P2
     if (d.K <= 2) MCEP_PK(2);
     if (d.K <= 4) MCEP_PK(4);
     if (d.K <= 8) MCEP_PK(8);

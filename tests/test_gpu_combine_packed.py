@@ -23,6 +23,11 @@ CASES = [
     EPConfig("k11", 4, 40, 2048, 32, 11, True),
     EPConfig("k16_bf16", 2, 20, 1024, 32, 16, False),
     EPConfig("one_rank", 1, 36, 1024, 6, 2, True),
+    # bf16 payloads with few rows per token: two 512-element chunks per lane, the second one partly or wholly
+    # beyond the hidden size in the last slab
+    EPConfig("k2_bf16", 8, 40, 4096, 8, 2, False, masked_fraction=0.1),
+    EPConfig("k4_h1536_bf16", 4, 20, 1536, 16, 4, False),
+    EPConfig("k1_h640_bf16", 2, 12, 640, 4, 1, False),
     EPConfig("masked_fp8", 8, 64, 1024, 8, 2, True, masked_fraction=0.3),
     EPConfig("zipf_outliers", 8, 32, 2048, 64, 8, True, routing="zipf", outlier_fraction=0.05),
     # slab counts on either side of the 8 XCDs the kernel's block order deals slabs to: 8, 9, 10 and 16 slabs of
@@ -74,6 +79,22 @@ def test_packed_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, with_
     h.combine()
     torch.cuda.synchronize()
     assert torch.equal(h.combined.cpu().view(torch.int16), got.view(torch.int16))
+
+
+@pytest.mark.parametrize("chunks", [1, 2])
+@pytest.mark.parametrize("direct", [1, 0], ids=["direct", "handle"])
+def test_packed_combine_bf16_chunks_per_lane(gpu_device, oracle, chunks, direct):
+    """One or two 16-byte chunks per lane (option combine_chunks; by default two up to top-4) are the same function."""
+    cfg = EPConfig("chunks_bf16", 4, 28, 2560, 16, 3, False, masked_fraction=0.2)
+    announce(f"packed combine of a bf16 payload, combine_chunks={chunks} direct={direct}")
+    data = generate(cfg, seed=25)
+    h = run_dispatch(cfg, data, poison=True, options={"combine_chunks": chunks, "combine_direct": direct})
+    factor = torch.arange(cfg.num_experts).float() * 0.1 + 1.0
+    h.alloc_combine_io()
+    h.combine_packed(factor)
+    torch.cuda.synchronize()
+    want = oracle_two_step(oracle, cfg, data, h.num_tokens, factor)
+    assert torch.equal(h.combined.cpu().view(torch.int16), want.view(torch.int16))
 
 
 @pytest.mark.parametrize("direct", [1, 0], ids=["direct", "handle"])
