@@ -642,7 +642,8 @@ def main():
                      "frac_back_to_back": round(kernels[dom]["bytes"] / kernels[dom]["us_back_to_back"] / 1e3
                                                 / HBM_PEAK_GBPS, 4),
                      "traffic": traffic, "traffic_measured_at_commit": traffic_at if traffic is not None else None,
-                     "traffic_summary_stale": (traffic_at is not None and not traffic_current) or None},
+                     # true: a summary exists but was measured on other kernel sources; null: no summary for this workload
+                     "traffic_summary_stale": (not traffic_current) if traffic_at is not None else None},
     }
     if not args.no_flushed:
         out["flushed"] = time_flushed(h, args.kernel_iters, alg)
