@@ -1,7 +1,8 @@
 """Seeded random worlds: odd rank / expert / top-k / hidden sizes, ragged token
 counts (some zero), masked tokens, ranks that take no part, per-rank views of
 inactive ranks.  Every case runs dispatch -> cast back -> combine through the C
-ABI and is compared with the oracle bit for bit."""
+ABI and is compared with the oracle bit for bit; the packed combine then has to
+give the same bits from dispatch's output."""
 import os
 import random
 
@@ -88,3 +89,9 @@ def test_random_world(gpu_device, oracle, seed):
     for r, n in enumerate(sent):
         assert torch.equal(got[r, :n].view(torch.int16), want[r, :n].view(torch.int16)), f"rank {r}"
         assert bool((got[r, n:] == 7.0).all()), f"rank {r}: rows beyond its tokens written"
+    # the combine fused with the consumer gives the same bits from dispatch's packed output
+    h.combined.fill_(7.0)
+    h.combine_packed(factor, present=present)
+    torch.cuda.synchronize()
+    fused = h.combined.cpu()
+    assert torch.equal(fused.view(torch.int16), got.view(torch.int16)), "packed combine differs from cast back + combine"
