@@ -95,7 +95,10 @@ int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
  * "combine_chunks", "combine_waves", "combine_nt", "packed_map": tuning knobs
  * for measurement sweeps; "fused_small": 1 (default) dispatches a world of at
  * most 8 ranks and "fused_small_max" (default 4096) selections in one kernel
- * launch, 0 always takes the count / pack / scale-transpose launches;
+ * launch - provided the ranks' index lists make at most "fused_small_rounds"
+ * rounds of 512 entries, each list counted by itself (default -1: 6 for an
+ * fp8 payload, 4 for bf16, which is where the launch stops paying) - and 0
+ * always takes the count / pack / scale-transpose launches;
  * "last_dispatch_launches", "last_combine_launches": read them to learn how
  * many kernels the world's last dispatch / combine call enqueued (a rank-table
  * upload counts); "fp8_arith": 0 (default) the fp8 scale arithmetic of the reference's

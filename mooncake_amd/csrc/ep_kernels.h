@@ -56,6 +56,7 @@ struct TableChunk {
 // The dispatch rank table of a small world, carried in kernel arguments: v[field * R + rank] with the
 // call's own R (at most kSmallRanks).
 constexpr int kSmallRanks = 8;
+constexpr int kSmallListRound = 512;  // index-list entries a wave of dispatch_small_kernel has in flight at a time
 struct SmallTable {
     uint64_t v[(int)DF_COUNT * kSmallRanks];
 };
@@ -152,6 +153,8 @@ struct Tuning {
     int comm_stream = 0;       // 1: per-rank rounds always run on the world's communication stream
     int fused_small = 1;       // dispatch of a small world (see dispatch_small_kernel) in one launch
     int fused_small_max = 4096;   // ... when the world names at most this many selections
+    int fused_small_rounds = -1;  // ... in at most this many rounds of kSmallListRound index-list entries, each rank's
+                                  // list counted by itself; -1: 6 for an fp8 payload, 4 for bf16 (measured)
     int last_dispatch_launches = 0;   // read-only in spirit: kernels the world's last dispatch / combine call enqueued
     int last_combine_launches = 0;    // (a rank-table upload counts; launches of other phases' calls do not)
     int blocking = 0;          // 1: a per-rank call returns only when its round has been launched (a thread per rank)

@@ -706,6 +706,7 @@ template <int KMAX>
 __device__ __forceinline__ void count_list(uint64_t list, int n, int E, const int (&ek)[KMAX], int (&cnt)[KMAX],
                                            int lane) {
     constexpr int kDepth = 4;             // 16-byte loads in flight per lane
+    static_assert(kDepth * 128 == kSmallListRound, "the host prices a world in rounds of this many entries");
     if ((list & 8) != 0 && n > 0) {
         // a list that starts in the middle of a 16-byte unit (rank r's slice of a rank-major tensor with an
         // odd number of entries per rank): its first entry by itself, pairs from there

@@ -525,7 +525,7 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         MC_ASSERT(recv_scales != nullptr);
     }
     int tgrid = 0;
-    long long selections = 0;
+    long long selections = 0, list_rounds = 0;
     // the rank table: on the stack, so that the allocation-free variant touches no heap either
     uint64_t tbl[(size_t)DF_COUNT * MC_EP_MAX_QP_COUNT];
     const size_t tbl_words = (size_t)DF_COUNT * R;
@@ -546,11 +546,16 @@ int world_dispatch_impl(mc_ep_world* w, const uint64_t* x, const uint64_t* topk_
         tbl[DF_NUM_TOKENS * R + r] = (uint64_t)num_tokens[r];
         if (num_tokens[r] > tgrid) tgrid = num_tokens[r];
         selections += (long long)num_tokens[r] * num_topk;
+        list_rounds += ((long long)num_tokens[r] * num_topk + kSmallListRound - 1) / kSmallListRound;
     }
     // A world that names few selections is dispatched in one launch, every wave rebuilding the routing it
     // needs from the index lists (dispatch_small_kernel); the rank table then travels in kernel arguments.
+    // What that costs grows with the rounds of index-list entries a late wave reads one after another (every
+    // rank's list is at least one round); measured against the launches it saves - two for an fp8 payload,
+    // one for bf16 - it pays up to six rounds and four.
+    const int rounds_limit = w->tuning.fused_small_rounds >= 0 ? w->tuning.fused_small_rounds : (use_fp8 ? 6 : 4);
     const bool fused = w->tuning.fused_small != 0 && phases == MC_EP_PHASE_ALL && R <= kSmallRanks && tgrid > 0 &&
-                       selections <= (long long)w->tuning.fused_small_max;
+                       selections <= (long long)w->tuning.fused_small_max && list_rounds <= (long long)rounds_limit;
     DeviceGuard guard(w->device);
     w->launches = 0;
     struct Tally {                                // the option "last_dispatch_launches", on every way out
@@ -1163,6 +1168,7 @@ static int* option_slot(Tuning& t, const char* name) {
     if (!strcmp(name, "last_combine_launches")) return &t.last_combine_launches;
     if (!strcmp(name, "fused_small")) return &t.fused_small;
     if (!strcmp(name, "fused_small_max")) return &t.fused_small_max;
+    if (!strcmp(name, "fused_small_rounds")) return &t.fused_small_rounds;
     if (!strcmp(name, "blocking")) return &t.blocking;
     if (!strcmp(name, "block_timeout_ms")) return &t.block_timeout_ms;
     if (!strcmp(name, "block_spin_us")) return &t.block_spin_us;

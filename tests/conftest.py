@@ -33,5 +33,8 @@ def fused_small(request):
     take the count / pack / scale-transpose launches like any other world (0)."""
     from tests import gpu_util
     gpu_util.DEFAULT_OPTIONS["fused_small"] = request.param
+    # (whatever the size rule of the default would say about a shape: the tests are about results)
+    gpu_util.DEFAULT_OPTIONS["fused_small_rounds"] = 1 << 20
     yield request.param
     gpu_util.DEFAULT_OPTIONS.pop("fused_small", None)
+    gpu_util.DEFAULT_OPTIONS.pop("fused_small_rounds", None)

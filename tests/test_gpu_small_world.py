@@ -9,6 +9,7 @@ import torch
 
 from mooncake_amd.harness import WorldHarness
 from mooncake_amd.workloads import EPConfig, generate
+from tests import gpu_util
 from tests.gpu_util import announce, compare_dispatch, run_dispatch
 
 pytestmark = pytest.mark.gpu
@@ -40,6 +41,40 @@ def ragged(cfg, on):
 
 def launches(h):
     return h.world.get_option("last_dispatch_launches")
+
+
+@pytest.fixture(autouse=True)
+def any_number_of_list_rounds(request):
+    """The default takes the one-launch dispatch only where it pays (few rounds of index-list entries); these
+    tests are about its results on every shape it accepts, so the rule is lifted - except where it is the subject."""
+    if "default_size_rule" in request.node.name:
+        yield
+        return
+    gpu_util.DEFAULT_OPTIONS["fused_small_rounds"] = 1 << 20
+    yield
+    gpu_util.DEFAULT_OPTIONS.pop("fused_small_rounds", None)
+
+
+def test_default_size_rule(gpu_device, oracle):
+    """One launch while the ranks' index lists make at most 6 rounds of 512 entries (fp8 payload: two launches
+    saved) or 4 (bf16: one), each rank's list counted by itself; the option moves the limit."""
+    announce("one-launch dispatch: the default size rule")
+    cases = [(EPConfig("fp8_6_rounds", 1, 384, 256, 16, 8, True), 1), (EPConfig("fp8_7_rounds", 1, 448, 256, 16, 8, True), 3),
+             (EPConfig("fp8_6_lists", 6, 8, 256, 12, 2, True), 1), (EPConfig("fp8_7_lists", 7, 8, 256, 14, 2, True), 3),
+             (EPConfig("bf16_4_rounds", 2, 128, 256, 16, 8, False), 1), (EPConfig("bf16_5_rounds", 5, 4, 256, 10, 2, False), 2)]
+    for cfg, want in cases:
+        data = generate(cfg, seed=47)
+        h = run_dispatch(cfg, data, poison=True)
+        assert (launches(h) == 1) == (want == 1), cfg.name
+        assert launches(h) >= want, cfg.name
+        ref = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, cfg.use_fp8)
+        compare_dispatch(h, ref, check_poison=True)
+    cfg = cases[1][0]
+    h = run_dispatch(cfg, generate(cfg, seed=47), poison=True, options={"fused_small_rounds": 7})
+    assert launches(h) == 1
+    cfg = cases[0][0]
+    h = run_dispatch(cfg, generate(cfg, seed=47), poison=True, options={"fused_small_rounds": 5})
+    assert launches(h) >= 3
 
 
 @pytest.mark.parametrize("cfg", CASES, ids=[c.name for c in CASES])
