@@ -92,7 +92,8 @@ int mc_ep_world_num_ranks(const mc_ep_world_t* world);
 int mc_ep_world_set_rank_silent(mc_ep_world_t* world, int rank, int silent);
 
 /* Options ("pack_waves", "pack_nt", "uniform", "routing_sum", "combine_direct",
- * "combine_chunks", "combine_waves", "combine_nt", "packed_map": tuning knobs
+ * "combine_chunks", "combine_waves", "combine_nt", "combine_occupancy",
+ * "packed_map": tuning knobs
  * for measurement sweeps; "fused_small": 1 (default) dispatches a world of at
  * most 8 ranks and "fused_small_max" (default 4096) selections in one kernel
  * launch - provided the ranks' index lists make at most "fused_small_rounds"

@@ -148,6 +148,7 @@ struct Tuning {
     int combine_chunks = 0;    // 16-byte chunks per lane in the combine kernel (1 or 2); 0: by top-k
     int combine_waves = 4;     // waves per block in the combine kernel
     int combine_nt = 3;        // bit 0: streaming loads, bit 1: streaming stores
+    int combine_occupancy = -1;   // waves of the combine kernel a CU runs at a time; 0: as many as fit, -1: by top-k
     int packed_map = 1;        // packed combine of an fp8 payload: 1 = slabs owned by XCDs, 0 = (rank, slab) groups per XCD
     int routing_sum = 1;       // allow the summed routing plan (see UnitPlan) where the shape permits
     int comm_stream = 0;       // 1: per-rank rounds always run on the world's communication stream

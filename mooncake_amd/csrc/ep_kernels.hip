@@ -1615,6 +1615,17 @@ hipError_t launch_count(const uint64_t* d_tbl, const RoutingScratch& sc, const D
 
 static int clamp_waves(int w) { return w < 1 ? 1 : (w > kMaxPackWaves ? kMaxPackWaves : w); }
 
+// Dynamic LDS a launch of wpb-wave blocks asks for (and never touches) so that a CU runs at most
+// `waves_per_cu` waves of it: floor(waves_per_cu / wpb) blocks fill the CU's LDS, at least one, at most what
+// 64 KiB per block allow without raising the kernel's limit.  0: no limit.
+static size_t occupancy_pad_bytes(int waves_per_cu, int wpb) {
+    constexpr size_t kCuLdsBytes = 160 * 1024, kMaxPad = 64 * 1024;
+    if (waves_per_cu <= 0) return 0;
+    const size_t blocks = waves_per_cu / wpb > 0 ? (size_t)(waves_per_cu / wpb) : 1;
+    const size_t pad = kCuLdsBytes / blocks / 1024 * 1024;
+    return pad > kMaxPad ? kMaxPad : pad;
+}
+
 static long long transpose_items(const Dims& d, int* parts_out) {
     const int G = d.H / 128;
     const int parts = (G + kTransposeGroups - 1) / kTransposeGroups;
@@ -1730,8 +1741,15 @@ static hipError_t launch_reduce_t(const ReduceLaunch& rl, const Dims& d, const T
     const int wpb = clamp_waves(t.combine_waves);
     const int blocks = (int)((total + wpb - 1) / wpb);
     const bool ntl = t.combine_nt & 1, nts = t.combine_nt & 2;
+    // Waves per CU.  With seven or more rows per token - 7 KB and more of loads in flight per wave - the
+    // kernel is fastest at 16 to 20 waves per CU: 1.5 to 4 % faster at top-8, depending on the machine, than at
+    // the 32 the hardware would run (fewer rows being walked at once), a little at top-11 and top-16; 12
+    // waves no longer cover the latency.  With fewer rows per wave it wants all 32 (top-3: 39.6 us against
+    // 41.1 at 20).  The limit is imposed with unused dynamic LDS: a CU's 160 KiB hold so many blocks and no more.
+    const int occupancy = t.combine_occupancy >= 0 ? t.combine_occupancy : (d.K >= 7 ? 20 : 0);
+    const size_t pad = occupancy_pad_bytes(occupancy, wpb);
 #define MCEP_REDUCE(A, B)                                                                                        \
-    hipLaunchKernelGGL((reduce_kernel<KMAX, CH, A, B, DIRECT>), dim3(blocks), dim3(wpb * 64), 0, stream, rl.d_tbl, \
+    hipLaunchKernelGGL((reduce_kernel<KMAX, CH, A, B, DIRECT>), dim3(blocks), dim3(wpb * 64), pad, stream, rl.d_tbl, \
                        rl.d_routes, rl.stamp, rl.sc, rl.src, rl.d_zero_row, d.R, d.E, d.K, d.max_tokens, d.H,    \
                        slabs, d.Tgrid, (int)total)
     if (ntl && nts) MCEP_REDUCE(true, true);

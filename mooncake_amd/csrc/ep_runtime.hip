@@ -1161,6 +1161,7 @@ static int* option_slot(Tuning& t, const char* name) {
     if (!strcmp(name, "combine_direct")) return &t.combine_direct;
     if (!strcmp(name, "combine_chunks")) return &t.combine_chunks;
     if (!strcmp(name, "packed_map")) return &t.packed_map;
+    if (!strcmp(name, "combine_occupancy")) return &t.combine_occupancy;
     if (!strcmp(name, "routing_sum")) return &t.routing_sum;
     if (!strcmp(name, "combine_waves")) return &t.combine_waves;
     if (!strcmp(name, "combine_nt")) return &t.combine_nt;

@@ -220,6 +220,25 @@ def test_combine_matches_oracle(gpu_device, oracle, cfg, is_ragged, chunks, cnt,
         assert bool((got[r, n:] == 7.0).all()), "rows beyond num_tokens written"
 
 
+@pytest.mark.parametrize("waves,occupancy", [(4, 0), (4, 20), (4, 8), (1, 20), (8, 20), (8, 4), (3, 200)])
+def test_combine_launch_shapes_match_oracle(gpu_device, oracle, waves, occupancy):
+    """Waves per block and the cap on waves per CU (imposed with unused dynamic LDS; by default 20 from top-7 up)
+    change how the combine kernel is launched, not what it computes."""
+    cfg = EPConfig("launch_shapes", 8, 48, 3072, 64, 8, False, masked_fraction=0.1)
+    announce(f"combine with combine_waves={waves} combine_occupancy={occupancy}")
+    data = generate(cfg, seed=6)
+    h = run_dispatch(cfg, data, poison=False, options={"combine_waves": waves, "combine_occupancy": occupancy})
+    h.alloc_combine_io()
+    h.fill_expert_out_from_recv(torch.arange(cfg.num_experts).float() * 0.1 + 1.0)
+    h.combined.fill_(7.0)
+    h.combine()
+    torch.cuda.synchronize()
+    ref_d = oracle.dispatch(data["x"], data["topk_idx"], h.num_tokens, cfg.max_tokens, cfg.num_experts, False)
+    want = oracle.combine(h.expert_out.cpu(), data["topk_idx"], data["topk_weights"], ref_d["src_info"],
+                          ref_d["layout_range"], h.num_tokens, cfg.max_tokens, cfg.num_experts, use_fma=True)
+    assert torch.equal(h.combined.cpu().view(torch.int16), want.view(torch.int16))
+
+
 @pytest.mark.parametrize("direct", [1, 0])
 def test_combine_skips_inactive_ranks(gpu_device, oracle, direct, fused_small):
     cfg = EPConfig("inactive", 4, 16, 1024, 16, 4, False)
