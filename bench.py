@@ -379,6 +379,18 @@ def stream_ceilings(cfg, S, iters):
     us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_gather_rows(
         dst.data_ptr(), layout.data_ptr(), H * 2, N, cfg.num_experts, region_rows, used, stream)), iters)
     record("gather 8:1 of scattered rows of the packed layout, reduce sized", us, 8 * N * H * 2, N * H * 2)
+    # the two gathers once more at the occupancy the combine kernel is launched with from top-7 up
+    _lib.check(lib.mc_ep_debug_set_stream_occupancy(20))
+    try:
+        us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_stream(4, dst.data_ptr(), layout.data_ptr(),
+                                                                          out_rows, stream)), iters)
+        record("gather 8:1, reduce sized, 20 waves per CU", us, 8 * out_rows, out_rows)
+        us = time_back_to_back(lambda: _lib.check(lib.mc_ep_debug_gather_rows(
+            dst.data_ptr(), layout.data_ptr(), H * 2, N, cfg.num_experts, region_rows, used, stream)), iters)
+        record("gather 8:1 of scattered rows of the packed layout, reduce sized, 20 waves per CU", us,
+               8 * N * H * 2, N * H * 2)
+    finally:
+        _lib.check(lib.mc_ep_debug_set_stream_occupancy(0))
     # and the 1 : 4 scatter on the geometry of the fp8 layout: every source row read once, written (at half its
     # size) to 8 whole rows at scattered places of [experts, ranks * max_tokens, hidden] bytes
     layout8 = layout.view(torch.uint8)[: cfg.num_experts * region_rows * H]

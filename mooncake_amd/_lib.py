@@ -89,6 +89,7 @@ SIGNATURES = {
 DEBUG_SIGNATURES = {
     "mc_ep_debug_copy": (c_int, [c_uint64, c_uint64, c_uint64, c_uint64]),
     "mc_ep_debug_stream": (c_int, [c_int, c_uint64, c_uint64, c_uint64, c_uint64]),
+    "mc_ep_debug_set_stream_occupancy": (c_int, [c_int]),
     "mc_ep_debug_gather_rows": (c_int, [c_uint64, c_uint64, c_int, c_int64, c_int, c_int64, c_int, c_uint64]),
     "mc_ep_debug_scatter_rows": (c_int, [c_uint64, c_uint64, c_int, c_int64, c_int, c_int64, c_int, c_uint64]),
 }

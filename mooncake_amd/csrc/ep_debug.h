@@ -29,6 +29,11 @@ int mc_ep_debug_copy(uint64_t dst_ptr, uint64_t src_ptr, uint64_t bytes, uint64_
  * src / dst must hold what the kind reads / writes. */
 int mc_ep_debug_stream(int kind, uint64_t dst_ptr, uint64_t src_ptr, uint64_t unit_bytes, uint64_t stream_ptr);
 
+/* From now on the synthetic streams (mc_ep_debug_stream, _gather_rows, _scatter_rows) run at most this many
+ * waves per CU (0, the default: as many as fit), so that a stream can be measured at the occupancy the
+ * kernel it stands for is launched with. */
+int mc_ep_debug_set_stream_occupancy(int waves_per_cu);
+
 /* The reduce kernel's address pattern with nothing else: out_rows rows of
  * row_bytes (multiple of 1024), each the xor of 8 whole rows at computed,
  * scattered places of a [regions, region_rows, row_bytes] source of which the

@@ -198,6 +198,8 @@ long long cast_back_chunks(long long max_rows, int num_experts);
 hipError_t launch_cast_back(const uint64_t* d_tbl, void* d_chunk_map, const float* d_factor, bool use_fp8,
                             long long max_rows, const Dims& d, hipStream_t stream);
 hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
+// waves per CU the synthetic streams run at from now on (0: as many as fit)
+void set_stream_occupancy(int waves_per_cu);
 // a synthetic stream of `unit_bytes / 16` threads with one of the data kernels' read : write mixes (see stream_kernel)
 hipError_t launch_stream(int kind, void* dst, const void* src, size_t unit_bytes, hipStream_t stream);
 // out_rows rows, each the xor of 8 rows scattered over a [regions, region_rows] layout (see stream_rows_kernel)

@@ -1869,7 +1869,13 @@ hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t str
     return hipGetLastError();
 }
 
+// waves per CU the synthetic streams below are held to (0: as many as fit), so that a stream can be measured
+// at the occupancy its kernel runs at
+static int g_stream_occupancy = 0;
+void set_stream_occupancy(int waves_per_cu) { g_stream_occupancy = waves_per_cu > 0 ? waves_per_cu : 0; }
+
 hipError_t launch_stream(int kind, void* dst, const void* src, size_t unit_bytes, hipStream_t stream) {
+    const size_t pad = occupancy_pad_bytes(g_stream_occupancy, 4);
     const size_t n = unit_bytes / 16;
     if (n == 0) return hipSuccess;
     const size_t blocks = (n + 255) / 256;
@@ -1878,12 +1884,12 @@ hipError_t launch_stream(int kind, void* dst, const void* src, size_t unit_bytes
     uint4* d = (uint4*)dst;
     const uint4* s = (const uint4*)src;
     switch (kind) {
-        case 0: hipLaunchKernelGGL(stream_kernel<0>, grid, block, 0, stream, d, s, n); break;
-        case 1: hipLaunchKernelGGL(stream_kernel<1>, grid, block, 0, stream, d, s, n); break;
-        case 2: hipLaunchKernelGGL(stream_kernel<2>, grid, block, 0, stream, d, s, n); break;
-        case 3: hipLaunchKernelGGL(stream_kernel<3>, grid, block, 0, stream, d, s, n); break;
-        case 4: hipLaunchKernelGGL(stream_kernel<4>, grid, block, 0, stream, d, s, n); break;
-        default: hipLaunchKernelGGL(stream_kernel<5>, grid, block, 0, stream, d, s, n); break;
+        case 0: hipLaunchKernelGGL(stream_kernel<0>, grid, block, pad, stream, d, s, n); break;
+        case 1: hipLaunchKernelGGL(stream_kernel<1>, grid, block, pad, stream, d, s, n); break;
+        case 2: hipLaunchKernelGGL(stream_kernel<2>, grid, block, pad, stream, d, s, n); break;
+        case 3: hipLaunchKernelGGL(stream_kernel<3>, grid, block, pad, stream, d, s, n); break;
+        case 4: hipLaunchKernelGGL(stream_kernel<4>, grid, block, pad, stream, d, s, n); break;
+        default: hipLaunchKernelGGL(stream_kernel<5>, grid, block, pad, stream, d, s, n); break;
     }
     return hipGetLastError();
 }
@@ -1896,7 +1902,8 @@ hipError_t launch_stream_rows(void* dst, const void* src, int row_bytes, long lo
     if (row_units % 64 != 0 || (long long)regions * used > 0x7fffffffll) return hipErrorInvalidValue;
     const size_t blocks = (n + 255) / 256;
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(stream_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)dst, (const uint4*)src,
+    hipLaunchKernelGGL(stream_rows_kernel, dim3((unsigned)blocks), dim3(256), occupancy_pad_bytes(g_stream_occupancy, 4),
+                       stream, (uint4*)dst, (const uint4*)src,
                        row_units, n, regions, (size_t)region_rows, used);
     return hipGetLastError();
 }
@@ -1909,7 +1916,8 @@ hipError_t launch_stream_rows_scatter(void* dst, const void* src, int row_bytes,
     if (row_units % 64 != 0 || (long long)regions * used > 0x7fffffffll) return hipErrorInvalidValue;
     const size_t blocks = (n + 255) / 256;
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(stream_rows_scatter_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)dst,
+    hipLaunchKernelGGL(stream_rows_scatter_kernel, dim3((unsigned)blocks), dim3(256),
+                       occupancy_pad_bytes(g_stream_occupancy, 4), stream, (uint4*)dst,
                        (const uint4*)src, row_units, n, regions, (size_t)region_rows, used);
     return hipGetLastError();
 }

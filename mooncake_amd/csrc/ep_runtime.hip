@@ -1624,6 +1624,12 @@ int mc_ep_hook_destroy(mc_ep_hook_t* h) {
     return MC_EP_OK;
 }
 
+int mc_ep_debug_set_stream_occupancy(int waves_per_cu) {
+    Lock lock(g_mu);
+    set_stream_occupancy(waves_per_cu);
+    return MC_EP_OK;
+}
+
 int mc_ep_debug_stream(int kind, uint64_t dst_ptr, uint64_t src_ptr, uint64_t unit_bytes, uint64_t stream_ptr) {
     MC_ASSERT(dst_ptr != 0 && src_ptr != 0 && unit_bytes % 16 == 0 && kind >= 0 && kind <= 5);
     MC_HIP(launch_stream(kind, (void*)dst_ptr, (const void*)src_ptr, (size_t)unit_bytes, (hipStream_t)stream_ptr));
