@@ -40,6 +40,7 @@ hipError_t launch_cast_back(const uint64_t*, void*, const float*, bool, long lon
     return launched(s);
 }
 hipError_t launch_copy(void*, const void*, size_t, hipStream_t s) { return launched(s); }
+void set_stream_occupancy(int) {}
 hipError_t launch_stream(int, void*, const void*, size_t, hipStream_t s) { return launched(s); }
 hipError_t launch_stream_rows(void*, const void*, int, long long, int, long long, int, hipStream_t s) {
     return launched(s);
