@@ -586,7 +586,7 @@ __device__ __forceinline__ uint4 quantise16(uint4 a, uint4 b, float* scale_inv) 
 // column-major output with coalesced stores (writing them there from here would
 // be 4-byte stores 16 KB apart).
 //   NATIVE  which of the reference's two statements of the scale arithmetic (see quantise16)
-template <bool NTL, bool NATIVE>
+template <bool NTL, bool NATIVE, bool NTS>
 __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restrict__ tbl,
                                                         RoutingScratch sc, DispatchSource src,
                                                         float* __restrict__ scale_stage, int R, int E, int K,
@@ -630,12 +630,12 @@ __global__ __launch_bounds__(512) void pack_fp8_kernel(const uint64_t* __restric
     for (int k = 0; k < K; ++k) {
         const uint64_t row = read_lane_u64(dst.row, k * sel_lanes);
         if (row == 0) continue;
-        if (active) store16<false>((void*)(row + elem0), out);
+        if (active) store16<NTS>((void*)(row + elem0), out);
     }
 }
 
 // bf16: plain row copy, two unit-stride 16-byte pieces per lane.
-template <bool NTL>
+template <bool NTL, bool NTS>
 __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restrict__ tbl,
                                                          RoutingScratch sc, DispatchSource src,
                                                          float* __restrict__ /*scale_stage*/, int R, int E, int K,
@@ -679,7 +679,7 @@ __global__ __launch_bounds__(512) void pack_bf16_kernel(const uint64_t* __restri
         if (row == 0) continue;
 #pragma unroll
         for (int p = 0; p < 2; ++p)
-            if (active[p]) store16<false>((void*)(row + off[p]), v[p]);
+            if (active[p]) store16<NTS>((void*)(row + off[p]), v[p]);
     }
 }
 
@@ -1653,19 +1653,29 @@ static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const RoutingS
 hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, float* scale_stage,
                        const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
                        hipStream_t stream) {
-    // measured: streaming loads pay when a token's row goes to many experts, not when it goes to a few
-    // (and streaming stores never did)
-    const bool ntl = t.pack_nt >= 0 ? (t.pack_nt & 1) != 0 : d.K > 4;
+    // Streaming hints (bit 0: loads, bit 1: stores).  Default: streaming loads when a token's row goes to many
+    // experts, ordinary stores.  Streaming stores with ordinary loads do win the back-to-back benchmark step for
+    // fp8 payloads and long bf16 rows (DeepSeek-V3 decode 146 against 149 us), but only there: after a cache
+    // flush - the reference's timing protocol - the dispatch loses 9 to 13 us with them (the payload can no
+    // longer wait in the memory-side cache), and a consumer that reads the payload next finds it in memory
+    // instead of that cache.  Both hints together always lose (+6 to +9 us).
+    const int nt = t.pack_nt >= 0 ? t.pack_nt : (d.K > 4 ? 1 : 0);
+    const bool ntl = (nt & 1) != 0, nts = (nt & 2) != 0;
     if (use_fp8 && scale_stage == nullptr) return hipErrorInvalidValue;
     hipError_t err = hipSuccess;
     if (run_pack) {
-#define MCEP_PF(A, B) launch_pack_t(pack_fp8_kernel<A, B>, d_tbl, sc, src, scale_stage, d, t, stream)
+#define MCEP_PF(A, B)                                                                                   \
+    (nts ? launch_pack_t(pack_fp8_kernel<A, B, true>, d_tbl, sc, src, scale_stage, d, t, stream)        \
+         : launch_pack_t(pack_fp8_kernel<A, B, false>, d_tbl, sc, src, scale_stage, d, t, stream))
+#define MCEP_PB(A)                                                                                      \
+    (nts ? launch_pack_t(pack_bf16_kernel<A, true>, d_tbl, sc, src, scale_stage, d, t, stream)          \
+         : launch_pack_t(pack_bf16_kernel<A, false>, d_tbl, sc, src, scale_stage, d, t, stream))
         if (!use_fp8)
-            err = ntl ? launch_pack_t(pack_bf16_kernel<true>, d_tbl, sc, src, scale_stage, d, t, stream)
-                      : launch_pack_t(pack_bf16_kernel<false>, d_tbl, sc, src, scale_stage, d, t, stream);
+            err = ntl ? MCEP_PB(true) : MCEP_PB(false);
         else
             err = ntl ? (t.fp8_arith == 1 ? MCEP_PF(true, true) : MCEP_PF(true, false))
                       : (t.fp8_arith == 1 ? MCEP_PF(false, true) : MCEP_PF(false, false));
+#undef MCEP_PB
 #undef MCEP_PF
     }
     if (err != hipSuccess || !use_fp8 || !run_finish) return err;

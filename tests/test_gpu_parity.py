@@ -62,7 +62,7 @@ def test_dispatch_matches_oracle(gpu_device, oracle, cfg, is_ragged, fused_small
     compare_dispatch(h, ref, check_poison=True)
 
 
-@pytest.mark.parametrize("nt", [0, 1])
+@pytest.mark.parametrize("nt", [0, 1, 2, 3])
 @pytest.mark.parametrize("uniform", [0, 1])
 @pytest.mark.parametrize("arith", [0, 1], ids=["torch_arith", "kernel_arith"])
 def test_fp8_pack_variants_match_oracle(gpu_device, oracle, nt, uniform, arith, fused_small):
@@ -80,7 +80,7 @@ def test_fp8_pack_variants_match_oracle(gpu_device, oracle, nt, uniform, arith, 
     compare_dispatch(h, ref, check_poison=True)
 
 
-@pytest.mark.parametrize("opts", [{"uniform": 0}, {"pack_waves": 1}, {"pack_waves": 8}, {"pack_nt": 1}, {"pack_nt": 0},
+@pytest.mark.parametrize("opts", [{"uniform": 0}, {"pack_waves": 1}, {"pack_waves": 8}, {"pack_nt": 1}, {"pack_nt": 0}, {"pack_nt": 2}, {"pack_nt": 3},
                                   {"routing_sum": 0}, {"routing_sum": 0, "uniform": 0}],
                          ids=lambda o: "-".join(f"{k}{v}" for k, v in o.items()))
 def test_dispatch_tuning_options_match_oracle(gpu_device, oracle, opts):
