@@ -53,6 +53,8 @@
 //                   counters are scaled against.
 #include "ep_kernels.h"
 
+#include <atomic>
+
 namespace mcep {
 
 namespace {
@@ -1881,11 +1883,14 @@ hipError_t launch_copy(void* dst, const void* src, size_t bytes, hipStream_t str
 
 // waves per CU the synthetic streams below are held to (0: as many as fit), so that a stream can be measured
 // at the occupancy its kernel runs at
-static int g_stream_occupancy = 0;
-void set_stream_occupancy(int waves_per_cu) { g_stream_occupancy = waves_per_cu > 0 ? waves_per_cu : 0; }
+static std::atomic<int> g_stream_occupancy{0};
+void set_stream_occupancy(int waves_per_cu) {
+    g_stream_occupancy.store(waves_per_cu > 0 ? waves_per_cu : 0, std::memory_order_relaxed);
+}
+static size_t stream_pad_bytes() { return occupancy_pad_bytes(g_stream_occupancy.load(std::memory_order_relaxed), 4); }
 
 hipError_t launch_stream(int kind, void* dst, const void* src, size_t unit_bytes, hipStream_t stream) {
-    const size_t pad = occupancy_pad_bytes(g_stream_occupancy, 4);
+    const size_t pad = stream_pad_bytes();
     const size_t n = unit_bytes / 16;
     if (n == 0) return hipSuccess;
     const size_t blocks = (n + 255) / 256;
@@ -1912,7 +1917,7 @@ hipError_t launch_stream_rows(void* dst, const void* src, int row_bytes, long lo
     if (row_units % 64 != 0 || (long long)regions * used > 0x7fffffffll) return hipErrorInvalidValue;
     const size_t blocks = (n + 255) / 256;
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(stream_rows_kernel, dim3((unsigned)blocks), dim3(256), occupancy_pad_bytes(g_stream_occupancy, 4),
+    hipLaunchKernelGGL(stream_rows_kernel, dim3((unsigned)blocks), dim3(256), stream_pad_bytes(),
                        stream, (uint4*)dst, (const uint4*)src,
                        row_units, n, regions, (size_t)region_rows, used);
     return hipGetLastError();
@@ -1927,7 +1932,7 @@ hipError_t launch_stream_rows_scatter(void* dst, const void* src, int row_bytes,
     const size_t blocks = (n + 255) / 256;
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
     hipLaunchKernelGGL(stream_rows_scatter_kernel, dim3((unsigned)blocks), dim3(256),
-                       occupancy_pad_bytes(g_stream_occupancy, 4), stream, (uint4*)dst,
+                       stream_pad_bytes(), stream, (uint4*)dst,
                        (const uint4*)src, row_units, n, regions, (size_t)region_rows, used);
     return hipGetLastError();
 }

@@ -1625,7 +1625,6 @@ int mc_ep_hook_destroy(mc_ep_hook_t* h) {
 }
 
 int mc_ep_debug_set_stream_occupancy(int waves_per_cu) {
-    Lock lock(g_mu);
     set_stream_occupancy(waves_per_cu);
     return MC_EP_OK;
 }
