@@ -1,4 +1,5 @@
-"""The five named workloads at their full size on the GPU.
+"""The five named workloads at their full size on the GPU, and two worlds with a payload too large for the
+memory-side cache.
 
 Each is compared with the oracle on its valid rows (the oracle finishes a
 whole world in about a second) and through size-independent properties:
@@ -10,16 +11,23 @@ import pytest
 import torch
 
 from mooncake_amd.harness import WorldHarness, valid_rows
-from mooncake_amd.workloads import CONFIG_ORDER, CONFIGS, generate
+from mooncake_amd.workloads import CONFIG_ORDER, CONFIGS, EPConfig, generate
 from tests import ref_checks as rc
 from tests.gpu_util import announce, compare_dispatch
 
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("name,summed", [(n, 1) for n in CONFIG_ORDER] + [("dsv3_decode", 0), ("mixtral", 0)])
+# two worlds whose payload is past what the pack kernel treats as cacheable (384 MiB and more: it is then written
+# with streaming stores and read with ordinary loads), one per payload type
+BEYOND_CACHE = {"beyond_cache_bf16": EPConfig("beyond_cache_bf16", 16, 256, 7168, 128, 8, False),
+                "beyond_cache_fp8": EPConfig("beyond_cache_fp8", 16, 512, 7168, 128, 8, True)}
+
+
+@pytest.mark.parametrize("name,summed", [(n, 1) for n in CONFIG_ORDER] + [("dsv3_decode", 0), ("mixtral", 0)] +
+                         [(n, 1) for n in BEYOND_CACHE])
 def test_named_config_full_size(gpu_device, oracle, name, summed):
-    cfg = CONFIGS[name]
+    cfg = CONFIGS[name] if name in CONFIGS else BEYOND_CACHE[name]
     announce(f"full size {cfg} routing_sum={summed}")
     data = generate(cfg, seed=0)
     R, T, E, K, L = cfg.num_ranks, cfg.tokens_per_rank, cfg.num_experts, cfg.num_topk, cfg.num_local_experts
