@@ -140,7 +140,7 @@ struct Dims {
 // Tuning knobs, settable at run time for measurement sweeps.
 struct Tuning {
     int pack_waves = 4;        // waves per block in the pack kernel
-    int pack_nt = -1;          // bit 0: streaming (nontemporal) loads, bit 1: streaming stores; -1: by top-k and payload size
+    int pack_nt = -1;          // bit 0: streaming (nontemporal) loads, bit 1: streaming stores; -1: loads by top-k
     int uniform = 1;           // take per-rank addresses from kernel arguments when tensors are evenly spaced
     int fp8_arith = 0;         // fp8 scale arithmetic: 0 = the reference's PyTorch statement as CPU PyTorch runs it,
                                // 1 = the reference kernel's own (see pack_fp8_kernel)

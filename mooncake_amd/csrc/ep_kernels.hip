@@ -1655,18 +1655,14 @@ static hipError_t launch_pack_t(Kern kern, const uint64_t* d_tbl, const RoutingS
 hipError_t launch_pack(const uint64_t* d_tbl, const RoutingScratch& sc, const DispatchSource& src, float* scale_stage,
                        const Dims& d, bool use_fp8, const Tuning& t, bool run_pack, bool run_finish,
                        hipStream_t stream) {
-    // Streaming hints (bit 0: loads, bit 1: stores).  Both together always lose (+6 to +9 us on the decode
-    // workloads).  A payload that fits the 256 MB memory-side cache is written with ordinary stores (and read
-    // with streaming loads when a token's row goes to many experts): streaming stores would win the back-to-back
-    // benchmark step by 2 % (DeepSeek-V3 decode 146 against 149 us), but after a cache flush - the reference's
-    // timing protocol - the dispatch loses 9 to 13 us with them, and a consumer that reads the payload next
-    // finds it in memory instead of that cache.  A payload of 1.5 times that cache and more cannot wait there
-    // anyway: it is written with streaming stores, read with ordinary loads, and the dispatch is 5 to 17 %
-    // faster for it, flushed (read-only) or not (8 x 1024 tokens, hidden 7168, top-8, bf16: 155 against 172 us).
-    const unsigned long long row_bytes = use_fp8 ? (unsigned long long)d.H + (unsigned long long)(d.H / 128) * 4
-                                                 : 2ull * (unsigned long long)d.H;
-    const bool beyond_cache = (unsigned long long)d.R * d.Tgrid * d.K * row_bytes >= 3ull * (128ull << 20);
-    const int nt = t.pack_nt >= 0 ? t.pack_nt : (beyond_cache ? 2 : (d.K > 4 ? 1 : 0));
+    // Streaming hints (bit 0: loads, bit 1: stores).  Default: streaming loads when a token's row goes to many
+    // experts, ordinary stores.  Both hints together always lose (+6 to +9 us on the decode workloads).
+    // Streaming stores with ordinary loads win in the steady state - 2 % of the DeepSeek-V3 decode step, 5 to
+    // 13 % of a dispatch whose payload is several times the 256 MB memory-side cache - but lose under the
+    // reference's timing protocol, a written cache flush before every timed call (8 x 1024 tokens, hidden 7168,
+    // top-8, bf16: 218 against 180 us), and a consumer that reads a cacheable payload next finds it in memory
+    // instead of that cache.  They are an option (pack_nt = 2), not the default.
+    const int nt = t.pack_nt >= 0 ? t.pack_nt : (d.K > 4 ? 1 : 0);
     const bool ntl = (nt & 1) != 0, nts = (nt & 2) != 0;
     if (use_fp8 && scale_stage == nullptr) return hipErrorInvalidValue;
     hipError_t err = hipSuccess;

@@ -18,8 +18,7 @@ from tests.gpu_util import announce, compare_dispatch
 pytestmark = pytest.mark.gpu
 
 
-# two worlds whose payload is past what the pack kernel treats as cacheable (384 MiB and more: it is then written
-# with streaming stores and read with ordinary loads), one per payload type
+# two worlds whose payload (470 and 484 MB) is well past the 256 MB memory-side cache, one per payload type
 BEYOND_CACHE = {"beyond_cache_bf16": EPConfig("beyond_cache_bf16", 16, 256, 7168, 128, 8, False),
                 "beyond_cache_fp8": EPConfig("beyond_cache_fp8", 16, 512, 7168, 128, 8, True)}
 
